@@ -245,20 +245,39 @@ int tl_model_batch_generate_greedy(tl_model* m, int n, const int* first_tokens_h
  *      bf16 matrices [out][in] and stay bf16 in HBM; the residual stream, norms, router, scores and caches are FP32. ------ */
 enum tl_mixer_kind {
   TL_MIXER_SWA = 0,         /* windowed attention over a key/value cache (softmax or sigmoid weights, optional rotation) */
-  TL_MIXER_DELTA = 1        /* gated delta rule with a decay per key channel: a recurrent state per head, no cache of keys */
+  TL_MIXER_DELTA = 1,       /* gated delta rule with a decay per key channel: a recurrent state per head, no cache of keys */
+  TL_MIXER_LATENT = 2,      /* attention over a cached latent: queries through a normalised latent, keys and values of all heads
+                               up-projected from one normalised latent per token, plus one rotated key part shared by the heads;
+                               the cache holds the latent and that part only (optionally another layer's, kv_from) */
+  TL_MIXER_GDELTA = 3       /* generalized delta rule: decay and removal rate per key channel,
+                               S <- diag(w) S - (a u)(u^T S) + k v^T with the unit key u, o = S^T r */
 };
-enum tl_mlp_kind { TL_MLP_NONE = 0, TL_MLP_MOE = 1, TL_MLP_DENSE = 2 }; /* none | routed experts (+ shared expert) | one gated unit */
+enum tl_mlp_kind {
+  TL_MLP_NONE = 0,
+  TL_MLP_MOE = 1,           /* routed experts (+ shared expert) */
+  TL_MLP_DENSE = 2,         /* one gated unit */
+  TL_MLP_UNIT = 3           /* W_down act(W_up h): no gate; act = tl_act_kind (shared_ff is its size) */
+};
+enum tl_act_kind {
+  TL_ACT_NONE = 0,
+  TL_ACT_XIELU = 1,         /* z > 0: P z^2 + z / 2; z <= 0: Q (e^z - 1 - z) + z / 2, with P = softplus(p), Q = 1/2 + softplus(q)
+                               from the two numbers of the tensor mlp.act */
+  TL_ACT_TANH = 2
+};
 enum tl_block_kind {
   TL_BLOCK_POST_NORM = 0,   /* x += N1(mixer(x)); x += N2(ff(x)): the sublayers read x, the norm is on their output */
-  TL_BLOCK_PARALLEL = 1     /* h = N1(x); x += mixer(h) + ff(h): one norm, both sublayers read its output */
+  TL_BLOCK_PARALLEL = 1,    /* h = N1(x); x += mixer(h) + ff(h): one norm, both sublayers read its output */
+  TL_BLOCK_PRE_NORM = 2     /* x += mixer(N1(x)); x += ff(N2(x)): a norm in front of each sublayer */
 };
 enum tl_norm_kind {
   TL_NORM_RMS_ONE_PLUS = 0, /* y / sqrt(mean(y^2) + eps) * (1 + w) */
-  TL_NORM_DYT = 1           /* tanh(alpha y) * w + b: elementwise, no mean or variance (tensors <name>, <name>.alpha, <name>.b) */
+  TL_NORM_DYT = 1,          /* tanh(alpha y) * w + b: elementwise, no mean or variance (tensors <name>, <name>.alpha, <name>.b) */
+  TL_NORM_LAYER = 2         /* (y - mean) / sqrt(var + eps) * w + b, var = mean of the squared deviations (tensors <name>, <name>.b) */
 };
 enum tl_attn_weight {
   TL_ATTN_SOFTMAX = 0,      /* weights normalised over the visible keys */
-  TL_ATTN_SIGMOID = 1       /* weight of a visible key = sigmoid(score + bias[head]); not normalised */
+  TL_ATTN_SIGMOID = 1,      /* weight of a visible key = sigmoid(score + bias[head]); not normalised */
+  TL_ATTN_SOFTMAX_SINK = 2  /* softmax with one more term in the denominator: a sink of score 0 that carries no value */
 };
 enum tl_qk_norm {
   TL_QK_NORM_NONE = 0,
@@ -307,6 +326,16 @@ typedef struct tl_layer_spec {
   int route;                /* tl_route_kind */
   int route_groups, route_keep;
   int shared_gate;          /* 1: the shared expert's output is multiplied by sigmoid(w_sg . h) (mlp.shared.sg) */
+  float q_temp_coef;        /* TL_MIXER_SWA, q_temp_every > 0: the query at position p is multiplied by */
+  int q_temp_every;         /*   1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) */
+  int q_rank, kv_rank;      /* TL_MIXER_LATENT: sizes of the query latent and of the cached key/value latent */
+  int rot_dim;              /* TL_MIXER_LATENT: rotated query/key dimensions per head behind the `dim` plain ones (the key's are
+                               shared by all heads); rot_dims <= rot_dim of them turn */
+  int kv_from;              /* TL_MIXER_LATENT: 1 + index of an EARLIER latent layer (with a projection of its own and the same
+                               kv_rank, rot_dim and rotation) whose cached latent and rotated key part this layer reads; 0: its own */
+  int head_gate;            /* TL_MIXER_LATENT: 1: head n's output is multiplied by sigmoid(W_g h)_n (mix.g, one row per head) */
+  float decay_scale;        /* TL_MIXER_GDELTA: decay = exp(-decay_scale * sigmoid(W_w2 tanh(W_w1 h) + w0)); decay_rank = rows of w1 */
+  int act;                  /* TL_MLP_UNIT: tl_act_kind */
 } tl_layer_spec;
 typedef struct tl_stack_config {
   int width, vocab, n_layers;
@@ -366,11 +395,36 @@ int tl_delta_rule(const float* q_dev, const float* k_dev, const float* v_dev, co
 int tl_gated_head_norm(float* o_dev, const float* gate_dev, const float* weight_dev, int num_tokens, int heads, int vdim,
                        float eps, void* stream);
 
+/* tl_window_attention over caches whose rows are k_ld / v_ld floats apart (0: kv_heads * dim, kv_heads * vdim); mode is a
+ * tl_attn_weight. A latent cache serves as both: keys = the whole row, values = its first vdim columns. */
+int tl_window_attention_rows(const float* q_dev, const float* k_cache_dev, const float* v_cache_dev, float* out_dev, int num_tokens,
+                             int start_pos, int heads, int kv_heads, int dim, int vdim, int k_ld, int v_ld, int window,
+                             int keep_first, float scale, int mode, const float* head_bias_dev, void* stream);
+/* out[t] = (x[t] - mean) / sqrt(var + eps) * w + b */
+int tl_layer_norm(const float* x_dev, const float* weight_dev, const float* bias_dev, float* out_dev, int num_tokens, int width,
+                  float eps, void* stream);
+/* tl_dense_matmul with an activation (tl_act_kind; p, q as the kind describes them, already transformed) on the output rows
+ * from act_from on */
+int tl_dense_matmul_act(const void* w_bf16_dev, int rows, int cols, const float* x_dev, float* y_dev, int num_tokens, int terms,
+                        int act, float act_p, float act_q, int act_from, void* stream);
+/* per head g < groups: Y[t][g * y_stride + r] = sum_c W[g][r][c] X[t][g * x_stride + c], W bf16 [groups][rows][cols]; X rows
+ * ldx, Y rows ldy floats apart. terms as tl_dense_matmul (0: one token, FP32) */
+int tl_dense_matmul_heads(const void* w_bf16_dev, int groups, int rows, int cols, const float* x_dev, int ldx, int x_stride,
+                          float* y_dev, int ldy, int y_stride, int num_tokens, int terms, void* stream);
+/* generalized delta rule, token by token. p [T][ld] holds the projections r | k | v (heads * dim each) | gate (unused here) |
+ * a (heads * dim), dw [T][heads * dim] the decay's pre-activation: w = exp(-decay_scale * sigmoid(dw + w0)),
+ * a = sigmoid(a + a_bias), u = k / sqrt(sum k^2 + 1e-6) per head; S <- diag(w) S - (a u)(u^T S) + k v^T; o = S^T r.
+ * state_dev [heads][dim (value)][dim (key)], updated in place; o [T][heads * dim]; scratch_dev: 3 * T * heads * dim + 2 * T * heads floats */
+int tl_general_delta(const float* p_dev, int ld, const float* dw_dev, const float* w0_dev, const float* a_bias_dev,
+                     float decay_scale, float* state_dev, float* o_dev, float* scratch_dev, int num_tokens, int heads, int dim,
+                     void* stream);
+
 int tl_model_create_stack(const tl_stack_config* cfg, tl_model** out);
 /* tensors by checkpoint name: embed, embed.norm, final.norm, head, l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,q.norm,k.norm,vmix,pb},
  * l<i>.mix.{q,k,v}.conv, l<i>.mix.{b,a1,a2,g1,g2,A_log,dt_bias,norm}, l<i>.mlp.router, l<i>.mlp.router.b,
- * l<i>.mlp.e<j>.{gate,up,down}, l<i>.mlp.shared.{gate,up,down,sg}, l<i>.mlp.{gate,up,down}; a Dynamic Tanh norm <n> also has
- * <n>.alpha and <n>.b. type: TL_BF16 (matrices and vectors) or TL_F32 (vectors). */
+ * l<i>.mlp.e<j>.{gate,up,down}, l<i>.mlp.shared.{gate,up,down,sg}, l<i>.mlp.{gate,up,down,act}; latent attention
+ * l<i>.mix.{dq,dq.norm,uq,dkv,dkv.norm,uk,uv,g,o}; generalized delta rule l<i>.mix.{r,k,v,g,a,a.b,w1,w2,w0,norm,o}; a Dynamic
+ * Tanh norm <n> also has <n>.alpha and <n>.b, a layer norm <n>.b. type: TL_BF16 (matrices and vectors) or TL_F32 (vectors). */
 int tl_model_set_tensor_named(tl_model* m, const char* name, int type, const long long* shape, int ndim, const void* host_data);
 /* a prompt, or a portion of one, at positions start_pos..: logits of the token rows listed in rows_host (ascending; NULL: the
  * last token when n_rows == 1, all tokens when n_rows == num_tokens) -> logits_host[n_rows][vocab]. The cache keeps what

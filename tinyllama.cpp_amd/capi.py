@@ -34,7 +34,9 @@ class LayerSpec(C.Structure):
                 ("attn_weight", C.c_int), ("values_are_keys", C.c_int), ("rot_dims", C.c_int), ("rot_base", C.c_float),
                 ("rot_factor", C.c_float), ("rot_original", C.c_float), ("rot_fast", C.c_float), ("rot_slow", C.c_float),
                 ("conv_taps", C.c_int), ("decay_rank", C.c_int), ("gate_rank", C.c_int), ("route", C.c_int),
-                ("route_groups", C.c_int), ("route_keep", C.c_int), ("shared_gate", C.c_int)]
+                ("route_groups", C.c_int), ("route_keep", C.c_int), ("shared_gate", C.c_int), ("q_temp_coef", C.c_float),
+                ("q_temp_every", C.c_int), ("q_rank", C.c_int), ("kv_rank", C.c_int), ("rot_dim", C.c_int),
+                ("kv_from", C.c_int), ("head_gate", C.c_int), ("decay_scale", C.c_float), ("act", C.c_int)]
 
 
 class StackConfig(C.Structure):
@@ -136,6 +138,13 @@ SIGNATURES = {
                          _fp, _fp, _vp],
     "tl_delta_rule": [_fp, _fp, _fp, _fp, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp],
     "tl_gated_head_norm": [_fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_float, _vp],
+    "tl_window_attention_rows": [_fp, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                 C.c_int, C.c_int, C.c_float, C.c_int, _fp, _vp],
+    "tl_layer_norm": [_fp, _fp, _fp, _fp, C.c_int, C.c_int, C.c_float, _vp],
+    "tl_dense_matmul_act": [_vp, C.c_int, C.c_int, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int, _vp],
+    "tl_dense_matmul_heads": [_vp, C.c_int, C.c_int, C.c_int, _fp, C.c_int, C.c_int, _fp, C.c_int, C.c_int, C.c_int, C.c_int,
+                              _vp],
+    "tl_general_delta": [_fp, C.c_int, _fp, _fp, _fp, C.c_float, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, _vp],
 }
 
 # include/tlhip_debug.h: measurement / diagnostic hooks (not part of the boundary)

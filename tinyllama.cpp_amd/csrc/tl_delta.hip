@@ -16,6 +16,17 @@
 //                since o = (g s) . q + u (k . q) -- are reduced together over the sixteen lanes with row-local lane swaps, so a
 //                token costs one reduction latency, not two. A decode step is the same kernel with one token.
 //   gated norm   o / rms(o) * w * sigmoid(gate) per head, in front of the output projection.
+//
+// A second recurrence lives here beside it, the generalized delta rule: a decay w and a removal rate a per head and key
+// channel, the unit key u = k / sqrt(sum k^2 + 1e-6),
+//
+//     S <- diag(w) S - (a u)(u^T S) + k v^T      (both terms read the old S);   o = S^T r
+//
+//   gdelta_pre   per token and head: w = exp(-decay_scale sigmoid(dw + w0)), u, a u = sigmoid(a + b_a) u, and the two
+//                products that do not touch the state, r . (a u) and r . k.
+//   gdelta_scan  the same column-per-16-lanes layout as delta_scan. With x = u . s and y = (w r) . s over the OLD column s,
+//                o_c = y - (r . a u) x + (r . k) v_c and s <- w s - (a u) x + k v_c: the two sums over the state are reduced
+//                together, so a token again costs one reduction latency.
 #include <math.h>
 
 #include "tl_bf16.h"
@@ -197,19 +208,166 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const DeltaScanArgs a) 
   }
 }
 
-// a wave per (token, head)
-__global__ __launch_bounds__(256) void gated_head_norm_kernel(float* __restrict__ o, const float* __restrict__ gate,
-                                                             const float* __restrict__ w, int n_heads_total, int vdim,
-                                                             float eps) {
+// a wave per (token, head); gate rows gate_ld floats apart; w_stride = vdim: weights of its own for every head, 0: shared
+__global__ __launch_bounds__(256) void gated_head_norm_kernel(float* __restrict__ o, const float* __restrict__ gate, int gate_ld,
+                                                             const float* __restrict__ w, int w_stride, int heads,
+                                                             int n_heads_total, int vdim, float eps) {
   const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (i >= n_heads_total) return;
+  const int t = i / heads, h = i - t * heads;
   float* x = o + (size_t)i * vdim;
-  const float* g = gate + (size_t)i * vdim;
+  const float* g = gate + (size_t)t * gate_ld + (size_t)h * vdim;
+  const float* wh = w + (size_t)h * w_stride;
   float ss = 0.0f;
   for (int d = lane; d < vdim; d += 64) ss += x[d] * x[d];
   ss = tl_wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
-  for (int d = lane; d < vdim; d += 64) x[d] = x[d] * inv * w[d] * sigmoidf_(g[d]);
+  for (int d = lane; d < vdim; d += 64) x[d] = x[d] * inv * wh[d] * sigmoidf_(g[d]);
+}
+
+// grid (T, heads): a workgroup of 128 threads owns one head of one token (dim <= 512: four channels a thread)
+__global__ __launch_bounds__(128) void gdelta_pre_kernel(const GDeltaPreArgs a) {
+  __shared__ float red[3][2];
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int hd = a.heads * a.dim;
+  const float* row = a.p + (size_t)t * a.ld;
+  const float* rp = row + (size_t)h * a.dim;
+  const float* kp = row + hd + (size_t)h * a.dim;
+  const float* ap = row + 4 * (size_t)hd + (size_t)h * a.dim;
+  const size_t o0 = (size_t)t * hd + (size_t)h * a.dim;
+  float kv[4], rv[4], av[4];
+  float ss = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int d = tid + 128 * j;
+    kv[j] = rv[j] = av[j] = 0.0f;
+    if (d >= a.dim) continue;
+    kv[j] = kp[d];
+    rv[j] = rp[d];
+    av[j] = sigmoidf_(ap[d] + a.a_bias[h * a.dim + d]);
+    ss += kv[j] * kv[j];
+    a.w[o0 + d] = expf(-a.decay_scale * sigmoidf_(a.dw[o0 + d] + a.w0[h * a.dim + d]));
+  }
+  ss = tl_wave_sum(ss);
+  if ((tid & 63) == 0) red[0][tid >> 6] = ss;
+  __syncthreads();
+  const float inv = 1.0f / sqrtf(red[0][0] + red[0][1] + 1e-6f);
+  float s_rau = 0.0f, s_rk = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int d = tid + 128 * j;
+    if (d >= a.dim) continue;
+    const float u = kv[j] * inv, au = av[j] * u;
+    a.u[o0 + d] = u;
+    a.au[o0 + d] = au;
+    s_rau += rv[j] * au;
+    s_rk += rv[j] * kv[j];
+  }
+  s_rau = tl_wave_sum(s_rau);
+  s_rk = tl_wave_sum(s_rk);
+  if ((tid & 63) == 0) {
+    red[1][tid >> 6] = s_rau;
+    red[2][tid >> 6] = s_rk;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    a.rau[(size_t)t * a.heads + h] = red[1][0] + red[1][1];
+    a.rk[(size_t)t * a.heads + h] = red[2][0] + red[2][1];
+  }
+}
+
+// E key channels per lane: dim <= 16 E. grid (vdim / 16 rounded up, heads), 256 threads; staging as in delta_scan_kernel
+// (five key-channel vectors per token here: r, k, w, u, a u).
+template <int E>
+__global__ __launch_bounds__(256) void gdelta_scan_kernel(const GDeltaScanArgs a) {
+  constexpr int TB = E == 16 ? 4 : E == 8 ? 8 : 16;  // tokens per stage (40 KB of LDS at most)
+  constexpr int DP = 16 * E;                           // padded key size
+  constexpr int NL = (TB * DP) / 256;                  // elements of each vector a thread stages
+  __shared__ __attribute__((aligned(16))) float sr_[2][TB][DP], sk_[2][TB][DP], sw_[2][TB][DP], su_[2][TB][DP], sa_[2][TB][DP];
+  __shared__ float sv_[2][TB][16], sc_[2][TB][2];
+  const int tid = threadIdx.x, sub = tid & 15, cl = tid >> 4;
+  const int col = blockIdx.x * 16 + cl, h = blockIdx.y;
+  const bool live = col < a.vdim;  // lanes of a column beyond vdim compute on zeros and store nothing
+  const int d0 = sub * E;
+  float* sp = a.state + ((size_t)h * a.vdim + (live ? col : 0)) * a.dim;
+  float s[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) s[e] = (live && d0 + e < a.dim) ? sp[d0 + e] : 0.0f;
+  const int hd = a.heads * a.dim;
+  const float* rp = a.r + (size_t)h * a.dim;
+  const float* kp = a.k + (size_t)h * a.dim;
+  const size_t c0 = (size_t)h * a.dim;
+  float rr[NL], rk[NL], rw[NL], ru[NL], ra[NL], rv, rc;
+  auto fetch = [&](int t0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int idx = i * 256 + tid, tt = idx / DP, d = idx % DP;
+      const bool in = t0 + tt < a.T && d < a.dim;
+      const size_t g = (size_t)(t0 + tt) * hd + c0 + d;
+      rr[i] = in ? rp[(size_t)(t0 + tt) * a.ld + d] : 0.0f;
+      rk[i] = in ? kp[(size_t)(t0 + tt) * a.ld + d] : 0.0f;
+      rw[i] = in ? a.w[g] : 0.0f;
+      ru[i] = in ? a.u[g] : 0.0f;
+      ra[i] = in ? a.au[g] : 0.0f;
+    }
+    const int tt = tid >> 4, c = blockIdx.x * 16 + (tid & 15);
+    rv = (tt < TB && t0 + tt < a.T && c < a.vdim) ? a.v[(size_t)(t0 + tt) * a.ld + (size_t)h * a.vdim + c] : 0.0f;
+    const int t2 = tid >> 1;  // threads 0 .. 2 TB - 1: (r . a u, r . k) of the stage's tokens
+    rc = (t2 < TB && t0 + t2 < a.T) ? ((tid & 1) ? a.rk : a.rau)[(size_t)(t0 + t2) * a.heads + h] : 0.0f;
+  };
+  auto stash = [&](int b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int idx = i * 256 + tid, tt = idx / DP, d = idx % DP;
+      sr_[b][tt][d] = rr[i];
+      sk_[b][tt][d] = rk[i];
+      sw_[b][tt][d] = rw[i];
+      su_[b][tt][d] = ru[i];
+      sa_[b][tt][d] = ra[i];
+    }
+    if ((tid >> 4) < TB) sv_[b][tid >> 4][tid & 15] = rv;
+    if ((tid >> 1) < TB) sc_[b][tid >> 1][tid & 1] = rc;
+  };
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  int b = 0;
+  for (int t0 = 0; t0 < a.T; t0 += TB, b ^= 1) {
+    const bool more = t0 + TB < a.T;
+    if (more) fetch(t0 + TB);  // in flight under this stage's tokens
+    const int nt = a.T - t0 < TB ? a.T - t0 : TB;
+    for (int tt = 0; tt < nt; ++tt) {
+      float rc_[E], kc[E], wc[E], uc[E], ac[E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        rc_[e] = sr_[b][tt][d0 + e];
+        kc[e] = sk_[b][tt][d0 + e];
+        wc[e] = sw_[b][tt][d0 + e];
+        uc[e] = su_[b][tt][d0 + e];
+        ac[e] = sa_[b][tt][d0 + e];
+      }
+      const float vc = sv_[b][tt][cl], rau = sc_[b][tt][0], rkk = sc_[b][tt][1];
+      float x = 0.0f, y = 0.0f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        x += uc[e] * s[e];
+        s[e] *= wc[e];
+        y += rc_[e] * s[e];
+      }
+      x = row16_sum(x);
+      y = row16_sum(y);
+#pragma unroll
+      for (int e = 0; e < E; ++e) s[e] += kc[e] * vc - ac[e] * x;
+      if (live && sub == 0) a.o[(size_t)(t0 + tt) * a.heads * a.vdim + (size_t)h * a.vdim + col] = y - rau * x + rkk * vc;
+    }
+    if (more) stash(b ^ 1);  // the other buffer: its last readers passed the barrier at the end of the stage before
+    __syncthreads();
+  }
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (d0 + e < a.dim) sp[d0 + e] = s[e];
+  }
 }
 
 }  // namespace
@@ -245,13 +403,83 @@ int tl_launch_delta_scan(const DeltaScanArgs& a, hipStream_t s) {
   return 0;
 }
 
-int tl_launch_gated_head_norm(float* o, const float* gate, const float* w, int T, int heads, int vdim, float eps, hipStream_t s) {
-  TL_REQUIRE(o && gate && w && T > 0 && heads > 0 && vdim > 0, "gated_head_norm: bad arguments");
+int tl_launch_gated_head_norm_rows(float* o, const float* gate, int gate_ld, const float* w, int w_per_head, int T, int heads,
+                                   int vdim, float eps, hipStream_t s) {
+  TL_REQUIRE(o && gate && w && T > 0 && heads > 0 && vdim > 0 && gate_ld >= heads * vdim, "gated_head_norm: bad arguments");
   const long long n = (long long)T * heads;
   TL_REQUIRE(n <= 0x7fffffffLL, "gated_head_norm: too many heads");
-  gated_head_norm_kernel<<<(unsigned)((n + 3) / 4), 256, 0, s>>>(o, gate, w, (int)n, vdim, eps);
+  gated_head_norm_kernel<<<(unsigned)((n + 3) / 4), 256, 0, s>>>(o, gate, gate_ld, w, w_per_head ? vdim : 0, heads, (int)n, vdim, eps);
   TL_HIP(hipGetLastError());
   return 0;
+}
+
+int tl_launch_gated_head_norm(float* o, const float* gate, const float* w, int T, int heads, int vdim, float eps, hipStream_t s) {
+  return tl_launch_gated_head_norm_rows(o, gate, heads * vdim, w, 0, T, heads, vdim, eps, s);
+}
+
+int tl_launch_gdelta_pre(const GDeltaPreArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.p && a.dw && a.w0 && a.a_bias && a.w && a.u && a.au && a.rau && a.rk && a.T > 0, "gdelta_pre: bad arguments");
+  TL_REQUIRE(a.heads > 0 && a.heads <= 65535 && a.dim > 0 && a.dim <= 512, "gdelta_pre: %d heads of size %d", a.heads, a.dim);
+  TL_REQUIRE(a.ld >= 5 * a.heads * a.dim, "gdelta_pre: row stride %d below %d", a.ld, 5 * a.heads * a.dim);
+  gdelta_pre_kernel<<<dim3(a.T, a.heads), 128, 0, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_gdelta_scan(const GDeltaScanArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.r && a.k && a.v && a.w && a.u && a.au && a.rau && a.rk && a.state && a.o && a.T > 0, "gdelta_scan: bad arguments");
+  TL_REQUIRE(a.heads > 0 && a.heads <= 65535 && a.dim > 0 && a.vdim > 0, "gdelta_scan: %d heads, sizes %d / %d", a.heads, a.dim, a.vdim);
+  TL_REQUIRE(a.dim <= 256, "gdelta_scan: key size %d above 256", a.dim);
+  const dim3 grid((a.vdim + 15) / 16, a.heads);
+  const int e = (a.dim + 15) / 16;
+  if (e <= 1) gdelta_scan_kernel<1><<<grid, 256, 0, s>>>(a);
+  else if (e <= 2) gdelta_scan_kernel<2><<<grid, 256, 0, s>>>(a);
+  else if (e <= 4) gdelta_scan_kernel<4><<<grid, 256, 0, s>>>(a);
+  else if (e <= 8) gdelta_scan_kernel<8><<<grid, 256, 0, s>>>(a);
+  else gdelta_scan_kernel<16><<<grid, 256, 0, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int tl_general_delta(const float* p_dev, int ld, const float* dw_dev, const float* w0_dev, const float* a_bias_dev,
+                                float decay_scale, float* state_dev, float* o_dev, float* scratch_dev, int num_tokens, int heads,
+                                int dim, void* stream) {
+  TL_REQUIRE(scratch_dev && num_tokens > 0 && heads > 0 && dim > 0, "tl_general_delta: bad arguments");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t n = (size_t)num_tokens * heads * dim, m = (size_t)num_tokens * heads;
+  GDeltaPreArgs p = {};
+  p.p = p_dev;
+  p.ld = ld;
+  p.dw = dw_dev;
+  p.w0 = w0_dev;
+  p.a_bias = a_bias_dev;
+  p.decay_scale = decay_scale;
+  p.T = num_tokens;
+  p.heads = heads;
+  p.dim = dim;
+  p.w = scratch_dev;
+  p.u = scratch_dev + n;
+  p.au = scratch_dev + 2 * n;
+  p.rau = scratch_dev + 3 * n;
+  p.rk = scratch_dev + 3 * n + m;
+  TL_TRY(tl_launch_gdelta_pre(p, s));
+  GDeltaScanArgs d = {};
+  d.r = p_dev;
+  d.k = p_dev + (size_t)heads * dim;
+  d.v = p_dev + 2 * (size_t)heads * dim;
+  d.ld = ld;
+  d.w = p.w;
+  d.u = p.u;
+  d.au = p.au;
+  d.rau = p.rau;
+  d.rk = p.rk;
+  d.state = state_dev;
+  d.o = o_dev;
+  d.T = num_tokens;
+  d.heads = heads;
+  d.dim = dim;
+  d.vdim = dim;
+  return tl_launch_gdelta_scan(d, s);
 }
 
 extern "C" int tl_delta_prepare(const float* p_dev, int ld, const float* a_dev, int num_tokens, int heads, int kv_heads, int dim,

@@ -57,6 +57,8 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
   if (t0 >= hi) return;
   const int f0 = blockIdx.x * BM;
   const unsigned short* W = a.w + (size_t)g * a.rows * a.cols;
+  const float* X = a.x + (size_t)g * a.x_gstride;  // (one product per head: the group picks its columns)
+  float* Y = a.y + (size_t)g * a.y_gstride;
   for (int i = tid; i < BN; i += 256) {
     const int it = t0 + i;
     int r = -1;
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
   const int wave = tid >> 6, lane = tid & 63, wm = wave & 1, wn = wave >> 1;
   const int lr = tid >> 2, lk = (tid & 3) * 8;  // this thread stages 8 consecutive k of rows lr + 64 i of both tiles
   const int K = a.cols;
-  const bool vec = (K & 7) == 0 && (a.ldx & 3) == 0 && ((size_t)a.x & 15) == 0 && ((size_t)W & 15) == 0;
+  const bool vec = (K & 7) == 0 && (a.ldx & 3) == 0 && ((size_t)X & 15) == 0 && ((size_t)W & 15) == 0;
   const unsigned short* wp[WM];
   const float* xp[WN];
   bool wok[WM], xok[WN];
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
   for (int j = 0; j < WN; ++j) {
     const int xr = xrow[lr + 64 * j];
     xok[j] = xr >= 0;
-    xp[j] = a.x + (size_t)(xok[j] ? xr : 0) * a.ldx;
+    xp[j] = X + (size_t)(xok[j] ? xr : 0) * a.ldx;
   }
   uint4 wreg[WM];
   float xreg[WN][8];
@@ -163,13 +165,13 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
     __syncthreads();
   }
   // C layout: lane holds token (lane & 31) of a 32 x 32 product, features (e / 4) * 8 + (lane >> 5) * 4 + (e & 3)
-  const bool v4 = (a.ldy & 3) == 0 && ((size_t)a.y & 15) == 0;
+  const bool v4 = (a.ldy & 3) == 0 && ((size_t)Y & 15) == 0;
 #pragma unroll
   for (int j = 0; j < WN; ++j) {
     const int it = t0 + (wn * WN + j) * 32 + (lane & 31);
     if (it >= hi) continue;
     const int orow = a.y_rows ? a.y_rows[it] : it;
-    float* yr = a.y + (size_t)orow * a.ldy;
+    float* yr = Y + (size_t)orow * a.ldy;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
 #pragma unroll
@@ -185,6 +187,11 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
         if (a.softcap > 0.0f) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) acc[i][j][gq * 4 + e] = a.softcap * tanhf(acc[i][j][gq * 4 + e] / a.softcap);
+        }
+        if (a.act) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (f + e >= a.act_from) acc[i][j][gq * 4 + e] = tl_act_apply(a.act, acc[i][j][gq * 4 + e], a.act_p, a.act_q);
         }
         if (v4 && f + 4 <= a.rows) {
           *reinterpret_cast<float4*>(yr + f) =
@@ -203,16 +210,24 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
 template <int RW>
 __global__ __launch_bounds__(256) void dense_gemv_kernel(const unsigned short* __restrict__ W, int rows, int cols,
                                                          const float* __restrict__ x, float* __restrict__ y, int vec,
-                                                         float softcap) {
+                                                         float softcap, const GemvActArgs act, int x_stride, int y_stride) {
   const int lane = threadIdx.x & 63;
   const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
   if (row0 >= rows) return;
+  // blockIdx.y: the head of a one-product-per-head launch (its matrix, its columns of x, its piece of y)
+  W += (size_t)blockIdx.y * rows * cols;
+  x += (size_t)blockIdx.y * x_stride;
+  y += (size_t)blockIdx.y * y_stride;
   float out[RW];
   tl_wave_dot_rows<RW>(W + (size_t)row0 * cols, (size_t)cols, rows - row0, x, cols, vec != 0, lane, out);
   if (lane == 0) {
 #pragma unroll
     for (int r = 0; r < RW; ++r)
-      if (row0 + r < rows) y[row0 + r] = softcap > 0.0f ? softcap * tanhf(out[r] / softcap) : out[r];
+      if (row0 + r < rows) {
+        float v = softcap > 0.0f ? softcap * tanhf(out[r] / softcap) : out[r];
+        if (act.act && row0 + r >= act.act_from) v = tl_act_apply(act.act, v, act.act_p, act.act_q);
+        y[row0 + r] = v;
+      }
   }
 }
 
@@ -224,7 +239,9 @@ int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s) {
   TL_REQUIRE(!a.x_rows || a.x_div >= 1, "dense gemm: x_div must be >= 1");
   TL_REQUIRE(!a.glu || (a.rows & 1) == 0, "dense gemm: gated pairs need an even number of rows (got %d)", a.rows);
   const int groups = a.groups > 0 ? a.groups : 1;
-  TL_REQUIRE(groups == 1 || a.group_off, "dense gemm: groups without group_off");
+  TL_REQUIRE(groups == 1 || a.group_off || (a.x_gstride > 0 && a.y_gstride > 0 && !a.x_rows && !a.y_rows),
+             "dense gemm: groups without group_off or per-head column strides");
+  TL_REQUIRE(!a.act || !a.glu, "dense gemm: an activation and a gated unit in one epilogue");
   // 128 x 128 tiles when there is enough of both sides to fill them (grouped launches: tokens per group on average)
   const long long per_group = a.group_off ? (long long)a.T / groups : a.T;
   // Measured at width 4096, chunks of 512 tokens: a dense launch has too few 128 x 128 tiles to fill 256 CUs (6144 x 512:
@@ -248,16 +265,33 @@ int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s) {
   return 0;
 }
 
-int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s, float softcap) {
-  TL_REQUIRE(w && x && y && rows > 0 && cols > 0, "dense gemv: bad arguments");
-  const int vec = (cols & 7) == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0;
+static int launch_gemv(const uint16_t* w, int groups, int rows, int cols, const float* x, int x_stride, float* y, int y_stride,
+                       float softcap, const GemvActArgs& act, hipStream_t s) {
+  TL_REQUIRE(w && x && y && rows > 0 && cols > 0 && groups > 0 && groups <= 65535, "dense gemv: bad arguments");
+  // 16-byte loads need every head's matrix and columns aligned as the first one's
+  const int vec = (cols & 7) == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0 &&
+                  (groups == 1 || ((x_stride & 3) == 0 && (((size_t)rows * cols) & 7) == 0));
   // rows per wave: as many as still leave every CU a few workgroups
   const int cus = tl_num_cus();
-  if (rows >= 16 * 4 * cus) dense_gemv_kernel<4><<<(rows + 15) / 16, 256, 0, s>>>(w, rows, cols, x, y, vec, softcap);
-  else if (rows >= 8 * 4 * cus) dense_gemv_kernel<2><<<(rows + 7) / 8, 256, 0, s>>>(w, rows, cols, x, y, vec, softcap);
-  else dense_gemv_kernel<1><<<(rows + 3) / 4, 256, 0, s>>>(w, rows, cols, x, y, vec, softcap);
+  const long long all = (long long)rows * groups;
+  if (all >= 16 * 4 * cus) dense_gemv_kernel<4><<<dim3((rows + 15) / 16, groups), 256, 0, s>>>(w, rows, cols, x, y, vec, softcap, act, x_stride, y_stride);
+  else if (all >= 8 * 4 * cus) dense_gemv_kernel<2><<<dim3((rows + 7) / 8, groups), 256, 0, s>>>(w, rows, cols, x, y, vec, softcap, act, x_stride, y_stride);
+  else dense_gemv_kernel<1><<<dim3((rows + 3) / 4, groups), 256, 0, s>>>(w, rows, cols, x, y, vec, softcap, act, x_stride, y_stride);
   TL_HIP(hipGetLastError());
   return 0;
+}
+
+int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s, float softcap) {
+  return launch_gemv(w, 1, rows, cols, x, 0, y, 0, softcap, GemvActArgs{}, s);
+}
+
+int tl_launch_dense_gemv_act(const uint16_t* w, int rows, int cols, const float* x, float* y, const GemvActArgs& act, hipStream_t s) {
+  return launch_gemv(w, 1, rows, cols, x, 0, y, 0, 0.0f, act, s);
+}
+
+int tl_launch_dense_gemv_heads(const uint16_t* w, int groups, int rows, int cols, const float* x, int x_stride, float* y,
+                               int y_stride, hipStream_t s) {
+  return launch_gemv(w, groups, rows, cols, x, x_stride, y, y_stride, 0.0f, GemvActArgs{}, s);
 }
 
 extern "C" int tl_dense_matmul(const void* w_bf16_dev, int rows, int cols, const float* x_dev, float* y_dev, int num_tokens,
@@ -277,5 +311,55 @@ extern "C" int tl_dense_matmul(const void* w_bf16_dev, int rows, int cols, const
   a.ldy = rows;
   a.T = num_tokens;
   a.terms = terms;
+  return tl_launch_dense_gemm(a, s);
+}
+
+extern "C" int tl_dense_matmul_act(const void* w_bf16_dev, int rows, int cols, const float* x_dev, float* y_dev, int num_tokens,
+                                   int terms, int act, float act_p, float act_q, int act_from, void* stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  TL_REQUIRE(act >= TL_ACT_NONE && act <= TL_ACT_TANH, "tl_dense_matmul_act: activation kind %d", act);
+  if (terms == 0) {
+    TL_REQUIRE(num_tokens == 1, "tl_dense_matmul_act: terms 0 (FP32 GEMV) takes one token, not %d", num_tokens);
+    return tl_launch_dense_gemv_act(static_cast<const uint16_t*>(w_bf16_dev), rows, cols, x_dev, y_dev,
+                                    GemvActArgs{act, act_from, act_p, act_q}, s);
+  }
+  DenseArgs a = {};
+  a.w = static_cast<const uint16_t*>(w_bf16_dev);
+  a.rows = rows;
+  a.cols = cols;
+  a.x = x_dev;
+  a.ldx = cols;
+  a.y = y_dev;
+  a.ldy = rows;
+  a.T = num_tokens;
+  a.terms = terms;
+  a.act = act;
+  a.act_from = act_from;
+  a.act_p = act_p;
+  a.act_q = act_q;
+  return tl_launch_dense_gemm(a, s);
+}
+
+extern "C" int tl_dense_matmul_heads(const void* w_bf16_dev, int groups, int rows, int cols, const float* x_dev, int ldx,
+                                     int x_stride, float* y_dev, int ldy, int y_stride, int num_tokens, int terms, void* stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (terms == 0) {
+    TL_REQUIRE(num_tokens == 1, "tl_dense_matmul_heads: terms 0 (FP32 GEMV) takes one token, not %d", num_tokens);
+    return tl_launch_dense_gemv_heads(static_cast<const uint16_t*>(w_bf16_dev), groups, rows, cols, x_dev, x_stride, y_dev,
+                                      y_stride, s);
+  }
+  DenseArgs a = {};
+  a.w = static_cast<const uint16_t*>(w_bf16_dev);
+  a.rows = rows;
+  a.cols = cols;
+  a.x = x_dev;
+  a.ldx = ldx;
+  a.y = y_dev;
+  a.ldy = ldy;
+  a.T = num_tokens;
+  a.terms = terms;
+  a.groups = groups;
+  a.x_gstride = x_stride;
+  a.y_gstride = y_stride;
   return tl_launch_dense_gemm(a, s);
 }

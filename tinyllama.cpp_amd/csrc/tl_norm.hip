@@ -63,6 +63,10 @@ __global__ __launch_bounds__(1024) void qkv_post_kernel(const QkvPostArgs a) {
     const float inv = 1.0f / sqrtf(sq / (float)a.qd + a.eps);
     for (int c = threadIdx.x; c < a.qd; c += blockDim.x) q[c] = q[c] * inv * a.q_norm[c];
   }
+  if (a.q_temp_every > 0) {  // query temperature: grows by the logarithm of the position, in steps of q_temp_every positions
+    const float f = 1.0f + a.q_temp_coef * logf((float)((pos + 1) / a.q_temp_every) + 1.0f);
+    for (int c = threadIdx.x; c < a.qd; c += blockDim.x) q[c] *= f;
+  }
   {
     const float inv = a.k_norm ? 1.0f / sqrtf(sk / (float)a.kd + a.eps) : 1.0f;
     float* kr = a.kc + (size_t)pos * a.kd;
@@ -140,6 +144,75 @@ __global__ __launch_bounds__(1024) void norm_rows_kernel(const float* __restrict
 
 constexpr int kMaxRowFloats = 16 * 1024;  // 64 KB of LDS for the staged row
 
+// ---- layer norm: mean, then the mean of the squared deviations, both over the row staged in LDS (two passes, FP32) ----------
+// row[] holds the input; every thread returns with (mean, 1 / sqrt(var + eps))
+__device__ __forceinline__ void ln_stats(const float* row, int width, float eps, float* red, float* mean, float* inv) {
+  float sm = 0.0f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) sm += row[c];
+  const float mu = block_sum(sm, red) / (float)width;
+  float sv = 0.0f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float d = row[c] - mu;
+    sv += d * d;
+  }
+  const float var = block_sum(sv, red) / (float)width;
+  *mean = mu;
+  *inv = 1.0f / sqrtf(var + eps);
+}
+
+__global__ __launch_bounds__(1024) void embed_ln_kernel(const unsigned short* __restrict__ table, int vocab, int width,
+                                                       const int* __restrict__ tokens, const LnParams emb, const LnParams next,
+                                                       float eps, float* __restrict__ x, float* __restrict__ h) {
+  extern __shared__ __attribute__((aligned(16))) float row[];
+  __shared__ float red[kMaxWaves];
+  const int t = blockIdx.x, tok = tokens[t];
+  const bool in = tok >= 0 && tok < vocab;
+  const unsigned short* e = table + (size_t)(in ? tok : 0) * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) row[c] = in ? __uint_as_float((unsigned)e[c] << 16) : 0.0f;
+  __syncthreads();
+  float mu, inv;
+  if (emb.w) {
+    ln_stats(row, width, eps, red, &mu, &inv);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) row[c] = (row[c] - mu) * inv * emb.w[c] + emb.b[c];  // own columns only
+    __syncthreads();
+  }
+  for (int c = threadIdx.x; c < width; c += blockDim.x) x[(size_t)t * width + c] = row[c];
+  if (!next.w) return;
+  ln_stats(row, width, eps, red, &mu, &inv);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) h[(size_t)t * width + c] = (row[c] - mu) * inv * next.w[c] + next.b[c];
+}
+
+__global__ __launch_bounds__(1024) void resid_ln_kernel(float* __restrict__ x, const float* __restrict__ a, int width,
+                                                       const LnParams next, float eps, float* __restrict__ h) {
+  extern __shared__ __attribute__((aligned(16))) float row[];
+  __shared__ float red[kMaxWaves];
+  const int t = blockIdx.x;
+  float* xr = x + (size_t)t * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = xr[c] + a[(size_t)t * width + c];
+    xr[c] = v;
+    row[c] = v;
+  }
+  if (!next.w) return;
+  __syncthreads();
+  float mu, inv;
+  ln_stats(row, width, eps, red, &mu, &inv);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) h[(size_t)t * width + c] = (row[c] - mu) * inv * next.w[c] + next.b[c];
+}
+
+__global__ __launch_bounds__(1024) void ln_rows_kernel(const float* __restrict__ x, int width, const int* __restrict__ rows,
+                                                      const LnParams p, float eps, float* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) float row[];
+  __shared__ float red[kMaxWaves];
+  const int i = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[i] : i) * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) row[c] = xr[c];
+  __syncthreads();
+  float mu, inv;
+  ln_stats(row, width, eps, red, &mu, &inv);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) out[(size_t)i * width + c] = (row[c] - mu) * inv * p.w[c] + p.b[c];
+}
+
 __device__ __forceinline__ float dyt_of(float x, float alpha, float w, float b) { return tanhf(alpha * x) * w + b; }
 
 // grid (column blocks of 256, T)
@@ -208,6 +281,40 @@ extern "C" int tl_dyt_norm(const float* x_dev, const float* alpha_dev, const flo
                            float* out_dev, int num_tokens, int width, void* stream) {
   DytParams p = {alpha_dev, weight_dev, bias_dev};
   return tl_launch_dyt_rows(x_dev, width, nullptr, num_tokens, p, out_dev, static_cast<hipStream_t>(stream));
+}
+
+int tl_launch_embed_ln(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, const LnParams& emb,
+                       const LnParams& next, float eps, float* x, float* h, hipStream_t s) {
+  TL_REQUIRE(table && tokens_dev && x && T > 0 && vocab > 0, "embed_ln: bad arguments");
+  TL_REQUIRE(width > 0 && width <= kMaxRowFloats, "embed_ln: width %d outside (0, %d]", width, kMaxRowFloats);
+  TL_REQUIRE((!emb.w || emb.b) && (!next.w || (next.b && h)), "embed_ln: a norm without its bias or output");
+  embed_ln_kernel<<<T, row_threads(T), sizeof(float) * width, s>>>(table, vocab, width, tokens_dev, emb, next, eps, x, h);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_resid_ln(float* x, const float* a, int T, int width, const LnParams& next, float eps, float* h, hipStream_t s) {
+  TL_REQUIRE(x && a && T > 0, "resid_ln: bad arguments");
+  TL_REQUIRE(width > 0 && width <= kMaxRowFloats, "resid_ln: width %d outside (0, %d]", width, kMaxRowFloats);
+  TL_REQUIRE(!next.w || (next.b && h), "resid_ln: a norm without its bias or output");
+  resid_ln_kernel<<<T, row_threads(T), sizeof(float) * width, s>>>(x, a, width, next, eps, h);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_ln_rows(const float* x, int width, const int* rows_dev, int n, const LnParams& p, float eps, float* out,
+                      hipStream_t s) {
+  TL_REQUIRE(x && out && p.w && p.b && n > 0, "ln_rows: bad arguments");
+  TL_REQUIRE(width > 0 && width <= kMaxRowFloats, "ln_rows: width %d outside (0, %d]", width, kMaxRowFloats);
+  ln_rows_kernel<<<n, row_threads(n), sizeof(float) * width, s>>>(x, width, rows_dev, p, eps, out);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int tl_layer_norm(const float* x_dev, const float* weight_dev, const float* bias_dev, float* out_dev, int num_tokens,
+                             int width, float eps, void* stream) {
+  return tl_launch_ln_rows(x_dev, width, nullptr, num_tokens, LnParams{weight_dev, bias_dev}, eps, out_dev,
+                           static_cast<hipStream_t>(stream));
 }
 
 int tl_launch_embed_norm(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, const float* w, float eps,

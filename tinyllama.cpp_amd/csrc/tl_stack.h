@@ -8,7 +8,10 @@
 //   tl_swa.hip    sliding-window attention without rotation, key and value sizes independent, over a flat FP32 cache
 //   tl_moe.hip    router (top-k, softmax over the chosen logits), grouping plan, clamped gated activation, decode GEMVs
 //   tl_norm.hip   RMS norms with zero-centred weights: embedding gather + norm, whole-projection q/k norm + value mixing +
-//                 cache write, residual += norm(sublayer output), row-gathering norm in front of the head
+//                 cache write, residual += norm(sublayer output), row-gathering norm in front of the head; layer norms of
+//                 pre-norm blocks (residual sum + the norm of the sublayer that follows)
+//   tl_rope.hip   rotary positions, per-head unit norm;  tl_delta.hip  two delta-rule recurrences with their preparation
+//   tl_latent.hip latent attention: norms of the latents, the rotated shared key part, cache rows, per-head output gate
 #pragma once
 #include "tl_internal.h"
 
@@ -33,10 +36,31 @@ struct DenseArgs {
   float glu_limit, glu_alpha;
   float glu_up_add;      // 1 in the formula above; a design may add something else (0: the plain gated unit)
   float softcap;         // > 0 (not with glu): y <- softcap * tanh(y / softcap)
+  // act != 0 (not with glu): a tl_act_kind on the output features from act_from on (TL_ACT_XIELU: act_p = softplus(p),
+  // act_q = 1/2 + softplus(q))
+  int act, act_from;
+  float act_p, act_q;
+  // groups > 1 without group_off: one product per head over ALL items -- group g multiplies matrix g with the columns
+  // x[.][g * x_gstride ..] and writes y[.][g * y_gstride ..]
+  int x_gstride, y_gstride;
 };
 int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s);
 // y[rows] = W x for one token, FP32 throughout (weights widened exactly)
 int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s, float softcap = 0.0f);
+struct GemvActArgs {
+  int act, act_from;     // as DenseArgs
+  float act_p, act_q;
+};
+int tl_launch_dense_gemv_act(const uint16_t* w, int rows, int cols, const float* x, float* y, const GemvActArgs& act, hipStream_t s);
+// one token, one product per head: y[g * y_stride + r] = W[g][r] . x[g * x_stride ..]
+int tl_launch_dense_gemv_heads(const uint16_t* w, int groups, int rows, int cols, const float* x, int x_stride, float* y,
+                               int y_stride, hipStream_t s);
+// the activation of tl_act_kind, for kernels that apply it themselves
+__host__ __device__ inline float tl_act_apply(int act, float z, float p, float q) {
+  if (act == TL_ACT_XIELU) return z > 0.0f ? p * z * z + 0.5f * z : q * (expm1f(z) - z) + 0.5f * z;
+  if (act == TL_ACT_TANH) return tanhf(z);
+  return z;
+}
 
 // ---- tl_swa.hip --------------------------------------------------------------------------------------------------------
 struct SwaArgs {
@@ -63,6 +87,11 @@ struct SwaArgs {
   // normalised over the keys; 0: softmax
   int sigmoid;
   const float* head_bias;
+  // sink != 0 (softmax only): the denominator has one more term, exp(0): a key of score 0 that carries no value
+  int sink;
+  // rows of the caches are kld / vld floats apart (0: kv_heads * dim, kv_heads * vdim): a cache of latent rows serves as
+  // keys (the whole row) and values (its first vdim columns) at once
+  int kld, vld;
 };
 int tl_launch_swa(const SwaArgs& a, hipStream_t s);
 int tl_swa_splits(int T, int window, int max_pos, int keep_first = 0);  // splits worth having for T tokens over a cache of max_pos rows
@@ -85,6 +114,9 @@ struct QkvPostArgs {
   int vmix;              // 0: v as it is; 1: this layer's v is kept in v_first; 2: v = (1 - lambda) v + lambda v_first
   float* v_first;        // [T][vd]
   const float* lambda;   // device scalar (vmix == 2)
+  // q_temp_every > 0: q at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)
+  float q_temp_coef;
+  int q_temp_every;
 };
 int tl_launch_qkv_post(const QkvPostArgs& a, hipStream_t s);
 // (declared here because the residual norm may carry it; the launcher is tl_moe.hip's)
@@ -144,6 +176,46 @@ int tl_launch_dyt_rows(const float* x, int width, const int* rows_dev, int n, co
 int tl_launch_norm_rows(const float* x, int width, const int* rows_dev, int n, const float* w, float eps, float* out,
                         hipStream_t s);
 
+// ---- layer norm (pre-norm blocks): (x - mean) / sqrt(var + eps) * w + b, statistics in FP32 over the row staged in LDS -------
+struct LnParams {
+  const float* w;        // [width] (NULL: no norm asked for)
+  const float* b;        // [width]
+};
+// x[t] = ln(embed[token[t]]; emb) (emb.w == NULL: the plain row); h[t] = ln(x[t]; next) when next.w is set
+int tl_launch_embed_ln(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, const LnParams& emb,
+                       const LnParams& next, float eps, float* x, float* h, hipStream_t s);
+// x[t] += a[t]; h[t] = ln(x[t]; next) when next.w is set (the norm in front of the sublayer that follows)
+int tl_launch_resid_ln(float* x, const float* a, int T, int width, const LnParams& next, float eps, float* h, hipStream_t s);
+// out[i] = ln(x[rows[i]]; p)   (rows == NULL: row i)
+int tl_launch_ln_rows(const float* x, int width, const int* rows_dev, int n, const LnParams& p, float eps, float* out,
+                      hipStream_t s);
+
+// ---- tl_latent.hip: what sits between the products of a latent-attention mixer ------------------------------------------
+struct LatentPostArgs {
+  float* p;              // [T][ld]: query latent (q_rank) | key/value latent (kv_rank) | rotated key part (rot_dim) | ...
+  int ld, q_rank, kv_rank, rot_dim;
+  const float* q_norm;   // plain weights [q_rank]: the query latent is RMS-normed in place
+  const float* kv_norm;  // plain weights [kv_rank] (NULL: this layer projects no latent of its own; kv_rank columns absent)
+  float eps;
+  int rot_dims;          // the first rot_dims of the rot_dim part turn, (2i, 2i + 1) by position * freq[i]
+  const double* freq;
+  float* cache;          // [max_pos][kv_rank + rot_dim]: row pos = normalised latent | rotated key part
+  int T, start_pos;
+  const int* pos_dev;
+};
+int tl_launch_latent_post(const LatentPostArgs& a, hipStream_t s);
+struct LatentQueryArgs {
+  const float* q;        // [T][heads * (dim + rot_dim)]: per head dim plain | rot_dim to be rotated
+  float* qa;             // [T][heads * (kv_rank + rot_dim)]: the rotated part goes behind each head's kv_rank absorbed columns
+  int heads, dim, rot_dim, kv_rank, rot_dims;
+  const double* freq;
+  int T, start_pos;
+  const int* pos_dev;
+};
+int tl_launch_latent_query(const LatentQueryArgs& a, hipStream_t s);
+// o[t][n][:] *= sigmoid(gate[t * gate_ld + n]) for the heads n of a token; o [T][heads * vdim]
+int tl_launch_head_gate(float* o, const float* gate, int gate_ld, int T, int heads, int vdim, hipStream_t s);
+
 // ---- tl_moe.hip --------------------------------------------------------------------------------------------------------
 int tl_launch_router(const RouterArgs& a, hipStream_t s);
 // slots (t * top + j) grouped by expert: off[experts + 1], slot_of[T * top]
@@ -195,6 +267,12 @@ struct RotaryArgs {
   const int* pos_dev;
 };
 int tl_launch_rotary(const RotaryArgs& a, hipStream_t s);
+// sin and cos of position * frequency: the product is formed and brought into [-pi, pi] in double, the functions are FP32
+__device__ __forceinline__ void tl_rotary_sincos(int pos, double freq, float* sn, float* cs) {
+  const double full = (double)pos * freq;
+  const float ang = (float)(full - 6.283185307179586476925 * rint(full * 0.159154943091895335769));
+  sincosf(ang, sn, cs);
+}
 
 // ---- tl_delta.hip ------------------------------------------------------------------------------------------------------
 struct DeltaPreArgs {
@@ -226,6 +304,37 @@ struct DeltaScanArgs {
 int tl_launch_delta_scan(const DeltaScanArgs& a, hipStream_t s);
 // o[t][h] <- o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t][h]) per head (w [vdim] shared by the heads); in place
 int tl_launch_gated_head_norm(float* o, const float* gate, const float* w, int T, int heads, int vdim, float eps, hipStream_t s);
+// the same with gate rows gate_ld floats apart and, w_per_head != 0, weights [heads * vdim] of their own for every head
+int tl_launch_gated_head_norm_rows(float* o, const float* gate, int gate_ld, const float* w, int w_per_head, int T, int heads,
+                                   int vdim, float eps, hipStream_t s);
+// ---- generalized delta rule: S <- diag(w) S - (a u)(u^T S) + k v^T (both terms read the old S), o = S^T r ------------------
+struct GDeltaPreArgs {
+  const float* p;        // [T][ld]: r | k | v | gate | a, heads * dim each (the gate is not read here)
+  int ld;
+  const float* dw;       // [T][heads * dim] pre-activation of the decay
+  const float* w0;       // [heads * dim]
+  const float* a_bias;   // [heads * dim]
+  float decay_scale;     // w = exp(-decay_scale * sigmoid(dw + w0))
+  int T, heads, dim;
+  float* w;              // out [T][heads * dim] decay
+  float* u;              // out [T][heads * dim] unit key k / sqrt(sum k^2 + 1e-6)
+  float* au;             // out [T][heads * dim] sigmoid(a + a_bias) * u
+  float* rau;            // out [T][heads] r . (a u)
+  float* rk;             // out [T][heads] r . k
+};
+int tl_launch_gdelta_pre(const GDeltaPreArgs& a, hipStream_t s);
+struct GDeltaScanArgs {
+  const float* r;        // token t, head h at r + t * ld + h * dim
+  const float* k;
+  const float* v;        // token t, head h at v + t * ld + h * vdim
+  int ld;
+  const float *w, *u, *au;  // [T][heads * dim]
+  const float *rau, *rk;    // [T][heads]
+  float* state;          // [heads][vdim][dim]: column c of head h's S, contiguous over the key channels; updated
+  float* o;              // [T][heads * vdim]
+  int T, heads, dim, vdim;
+};
+int tl_launch_gdelta_scan(const GDeltaScanArgs& a, hipStream_t s);
 
 // ---- tl_stack.hip: the engine ------------------------------------------------------------------------------------------
 struct TlStack;

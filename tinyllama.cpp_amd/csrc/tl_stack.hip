@@ -4,6 +4,8 @@
 // step can be captured into a hipGraph by tl_model.hip like the Llama step), T > 1 a chunk of a prompt (MFMA GEMMs).
 //
 // Blocks  TL_BLOCK_POST_NORM  x += norm1(mixer(x)); x += norm2(ff(x))   -- the sublayers read x itself, RMS norm on their OUTPUT
+//         TL_BLOCK_PRE_NORM   x += mixer(norm1(x)); x += ff(norm2(x))   -- a layer norm in FRONT of each sublayer; the launch that
+//                             finishes x also writes the norm of whatever reads x next (norm2, or the next layer's norm1)
 //         TL_BLOCK_PARALLEL   h = norm1(x); x += mixer(h) + ff(h)       -- one Dynamic Tanh norm, both sublayers read its output;
 //                             the norm of the NEXT block rides in the launch that finishes x (it is elementwise)
 // Mixers  TL_MIXER_SWA    q | k (| v) = W h in one product; either the whole-projection q/k RMS norm with optional value mixing
@@ -12,7 +14,15 @@
 //                         the first keys kept visible (tl_swa.hip); W_o
 //         TL_MIXER_DELTA  q | k | v | beta | a1 | g1 = W h in one product, a2 and g2 behind a1 and g1; convolution, unit norms
 //                         and decay (delta_pre), the recurrence over a per-head state (delta_scan), gated head norm; W_o
-// Feed-forward  TL_MLP_MOE  router (two kinds, tl_moe.hip) -> top experts (gated units) + optional shared expert, optionally
+//         TL_MIXER_LATENT query latent | key/value latent | rotated shared key part | head gates = W h in one product; norms,
+//                         rotation and the cache row (tl_latent.hip); queries up-projected, their plain part absorbed through
+//                         W_uk^T per head; attention over the cached latent rows themselves (tl_swa.hip, one "head" of keys whose
+//                         values are the first kv_rank columns); W_uv per head, head gates, W_o. A layer may read an earlier
+//                         latent layer's cache (kv_from) and then projects no latent of its own
+//         TL_MIXER_GDELTA r | k | v | gate | a | w1 = W h in one product (tanh on the w1 rows in its epilogue), w2 behind w1;
+//                         gdelta_pre, gdelta_scan over a per-head state, gated head norm with weights per head; W_o
+// Feed-forward  TL_MLP_UNIT  W_down act(W_up h), the activation in the first product's epilogue (pre-norm blocks)
+//               TL_MLP_MOE  router (two kinds, tl_moe.hip) -> top experts (gated units) + optional shared expert, optionally
 //                           gated per token;  TL_MLP_DENSE  one gated unit (it runs where a shared expert would)
 // A layer may use an earlier layer's tensors (weights_of) with a cache or state of its own.
 // The residual stream, norms, router, attention scores, caches and states are FP32; matrix operands of a prompt chunk are bf16
@@ -20,7 +30,8 @@
 //
 // Cache and state: one allocation. Attention layers: K [max_positions][kv_heads * dim] and V [max_positions][kv_heads * vdim],
 // flat by absolute position; a window only bounds what attention reads. Delta layers: S [heads][vdim][dim] and the
-// convolution's last taps - 1 inputs. tl_stack_reset gives everything back (one sequence at a time): zeros are the state of
+// convolution's last taps - 1 inputs; latent layers with a projection of their
+// own: rows [max_positions][kv_rank + rot_dim]; generalized delta layers: S [heads][dim][dim]. tl_stack_reset gives everything back (one sequence at a time): zeros are the state of
 // an empty sequence.
 #include <math.h>
 #include <stdio.h>
@@ -54,6 +65,17 @@ struct Layer {
   float* router_b = nullptr;
   float *kc = nullptr, *vc = nullptr;        // attention: caches
   float *state = nullptr, *hist = nullptr;   // delta rule: S and the convolution's history
+  float *norm2_b = nullptr;                  // layer norm
+  // latent attention: wqkv = dq | dkv | g stacked; wuq [heads * (dim + rot_dim)][q_rank]; wukt [heads][kv_rank][dim] (the
+  // TRANSPOSE of each head's block of mix.uk: the query is absorbed through it); wuv [heads][vdim][kv_rank] as stored
+  uint16_t *wuq = nullptr, *wukt = nullptr, *wuv = nullptr;
+  float *dq_norm = nullptr, *dkv_norm = nullptr;
+  float* ckv = nullptr;                      // cache rows [max_pos][kv_rank + rot_dim] (an owner's; kv_src's otherwise)
+  int kv_src = -1;                           // the latent layer whose cache this one reads (itself unless kv_from)
+  int gate_off = 0;                          // column of the head gates in the first product
+  // generalized delta rule: wqkv = r | k | v | g | a | w1 stacked, wa2 = w2
+  float *w0 = nullptr, *a_bias = nullptr;
+  float act_p = 0.0f, act_q = 0.0f;          // TL_MLP_UNIT: the activation's two numbers, transformed (tl_act_kind)
   std::set<std::string> expect, optional;    // tensor names (without the "l<i>." prefix) still missing / accepted and ignored
 };
 
@@ -63,7 +85,7 @@ struct TlStack {
   tl_stack_config cfg;
   std::vector<Layer> layers;
   uint16_t *embed = nullptr, *head = nullptr;
-  float *embed_norm = nullptr, *final_norm = nullptr, *final_b = nullptr, *final_alpha = nullptr;
+  float *embed_norm = nullptr, *embed_norm_b = nullptr, *final_norm = nullptr, *final_b = nullptr, *final_alpha = nullptr;
   int got_globals = 0, need_globals = 0;
   std::vector<void*> allocs;
   bool finalized = false;
@@ -84,6 +106,9 @@ struct TlStack {
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *proj = nullptr, *v_first = nullptr, *xn = nullptr;
   float* h = nullptr;       // norm-first blocks: the normalised input both sublayers read
   float *dq = nullptr, *da = nullptr, *dg = nullptr, *dbeta = nullptr, *ddecay = nullptr;  // delta rule
+  float *lq = nullptr, *lqa = nullptr;      // latent attention: up-projected queries, absorbed queries
+  float *gw = nullptr, *gu = nullptr, *gau = nullptr, *grau = nullptr, *grk = nullptr;  // generalized delta rule (gdelta_pre)
+  int max_lq = 0, max_lqa = 0, max_gd = 0, gdelta_layers = 0;
   float *act_buf = nullptr, *eout = nullptr, *sact = nullptr, *sout = nullptr, *sgate = nullptr;
   float* wts = nullptr;
   float* swa_ws = nullptr;  // partial results of split attention launches (few tokens, long windows)
@@ -152,7 +177,8 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
   TL_REQUIRE(cfg && out && cfg->layers, "tl_stack_create: null argument");
   TL_REQUIRE(cfg->width > 0 && cfg->vocab > 0 && cfg->n_layers > 0 && cfg->max_positions > 0,
              "tl_stack_create: non-positive size in the configuration");
-  TL_REQUIRE(cfg->norm == TL_NORM_RMS_ONE_PLUS || cfg->norm == TL_NORM_DYT, "tl_stack_create: norm kind %d", cfg->norm);
+  TL_REQUIRE(cfg->norm == TL_NORM_RMS_ONE_PLUS || cfg->norm == TL_NORM_DYT || cfg->norm == TL_NORM_LAYER,
+             "tl_stack_create: norm kind %d", cfg->norm);
   TlStack* st = new TlStack();
   st->cfg = *cfg;
   st->layers.resize(cfg->n_layers);
@@ -174,19 +200,27 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
     Layer& L = st->layers[i];
     L.sp = cfg->layers[i];
     const tl_layer_spec& sp = L.sp;
-    const bool dyt = cfg->norm == TL_NORM_DYT;
-    CREATE_REQUIRE(sp.mixer == TL_MIXER_SWA || sp.mixer == TL_MIXER_DELTA,
-                   "tl_stack_create: layer %d has mixer kind %d; this engine has windowed attention (%d) and the gated delta rule (%d)",
-                   i, sp.mixer, TL_MIXER_SWA, TL_MIXER_DELTA);
+    const bool dyt = cfg->norm == TL_NORM_DYT, lnorm = cfg->norm == TL_NORM_LAYER;
+    CREATE_REQUIRE(sp.mixer >= TL_MIXER_SWA && sp.mixer <= TL_MIXER_GDELTA,
+                   "tl_stack_create: layer %d has mixer kind %d; this engine has windowed attention (%d), the gated delta rule (%d), "
+                   "latent attention (%d) and the generalized delta rule (%d)",
+                   i, sp.mixer, TL_MIXER_SWA, TL_MIXER_DELTA, TL_MIXER_LATENT, TL_MIXER_GDELTA);
     CREATE_REQUIRE(sp.heads > 0 && sp.kv_heads > 0 && sp.heads % sp.kv_heads == 0 && sp.dim > 0 && sp.vdim > 0,
                    "tl_stack_create: layer %d: %d heads / %d key-value heads / sizes %d, %d", i, sp.heads, sp.kv_heads, sp.dim, sp.vdim);
-    CREATE_REQUIRE((sp.block == TL_BLOCK_POST_NORM && !dyt) || (sp.block == TL_BLOCK_PARALLEL && dyt),
+    CREATE_REQUIRE((sp.block == TL_BLOCK_POST_NORM && !dyt && !lnorm) || (sp.block == TL_BLOCK_PARALLEL && dyt) ||
+                       (sp.block == TL_BLOCK_PRE_NORM && lnorm),
                    "tl_stack_create: layer %d: block kind %d with norm kind %d (post-norm blocks take the RMS norm, parallel "
-                   "blocks the Dynamic Tanh norm)", i, sp.block, cfg->norm);
-    CREATE_REQUIRE(sp.mlp == TL_MLP_NONE || sp.mlp == TL_MLP_MOE || sp.mlp == TL_MLP_DENSE,
-                   "tl_stack_create: layer %d has feed-forward kind %d", i, sp.mlp);
+                   "blocks the Dynamic Tanh norm, pre-norm blocks the layer norm)", i, sp.block, cfg->norm);
+    CREATE_REQUIRE(sp.mlp >= TL_MLP_NONE && sp.mlp <= TL_MLP_UNIT, "tl_stack_create: layer %d has feed-forward kind %d", i, sp.mlp);
     CREATE_REQUIRE(sp.mlp != TL_MLP_DENSE || sp.block == TL_BLOCK_PARALLEL, "tl_stack_create: layer %d: a dense feed-forward "
                    "runs in parallel blocks only", i);
+    CREATE_REQUIRE(sp.mlp == TL_MLP_NONE || (sp.mlp == TL_MLP_UNIT) == (sp.block == TL_BLOCK_PRE_NORM),
+                   "tl_stack_create: layer %d: feed-forward kind %d in block kind %d (pre-norm blocks take the plain up / "
+                   "activation / down unit, and only they)", i, sp.mlp, sp.block);
+    CREATE_REQUIRE((sp.mixer != TL_MIXER_LATENT && sp.mixer != TL_MIXER_GDELTA) || sp.block == TL_BLOCK_PRE_NORM,
+                   "tl_stack_create: layer %d: latent attention and the generalized delta rule run in pre-norm blocks only", i);
+    CREATE_REQUIRE(sp.mixer != TL_MIXER_DELTA || sp.block == TL_BLOCK_PARALLEL, "tl_stack_create: layer %d: the delta rule runs "
+                   "in parallel blocks only", i);
     L.wsrc = i;
     if (sp.weights_of > 0) {
       CREATE_REQUIRE(sp.weights_of - 1 < i, "tl_stack_create: layer %d takes its tensors from layer %d, which is not an earlier "
@@ -203,9 +237,13 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
       CREATE_REQUIRE(sp.rot_dims >= 0 && sp.rot_dims <= sp.dim && (sp.rot_dims & 1) == 0 && (sp.rot_dims == 0 || sp.rot_base > 0.0f),
                      "tl_stack_create: layer %d: %d rotating dimensions of %d, base %g", i, sp.rot_dims, sp.dim, sp.rot_base);
       CREATE_REQUIRE(sp.keep_first >= 0, "tl_stack_create: layer %d: %d kept first keys", i, sp.keep_first);
+      CREATE_REQUIRE(sp.attn_weight >= TL_ATTN_SOFTMAX && sp.attn_weight <= TL_ATTN_SOFTMAX_SINK && sp.q_temp_every >= 0,
+                     "tl_stack_create: layer %d: attention weights of kind %d, query temperature every %d", i, sp.attn_weight,
+                     sp.q_temp_every);
       L.rotary_path = sp.rot_dims > 0 || sp.qk_norm == TL_QK_NORM_HEAD_UNIT || sp.values_are_keys;
-      CREATE_REQUIRE(!L.rotary_path || (sp.qk_norm != TL_QK_NORM_WHOLE && !sp.v_mix), "tl_stack_create: layer %d: rotation / "
-                     "per-head norm / values-are-keys do not combine with the whole-projection norm or value mixing", i);
+      CREATE_REQUIRE(!L.rotary_path || (sp.qk_norm != TL_QK_NORM_WHOLE && !sp.v_mix && sp.q_temp_every == 0),
+                     "tl_stack_create: layer %d: rotation / per-head norm / values-are-keys do not combine with the "
+                     "whole-projection norm, value mixing or a query temperature", i);
       CREATE_REQUIRE(sp.qk_norm >= TL_QK_NORM_NONE && sp.qk_norm <= TL_QK_NORM_HEAD_UNIT, "tl_stack_create: layer %d: q/k norm %d", i, sp.qk_norm);
       L.qd = sp.heads * sp.dim;
       L.kd = sp.kv_heads * sp.dim;
@@ -245,8 +283,71 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
           }
         }
       }
+    } else if (sp.mixer == TL_MIXER_LATENT) {
+      CREATE_REQUIRE(sp.q_rank > 0 && sp.kv_rank > 0 && sp.rot_dim >= 0 && sp.rot_dims >= 0 && sp.rot_dims <= sp.rot_dim &&
+                         (sp.rot_dims & 1) == 0 && (sp.rot_dims == 0 || sp.rot_base > 0.0f) && sp.kv_heads == sp.heads,
+                     "tl_stack_create: layer %d: latents of %d / %d, %d rotated dimensions of which %d turn (base %g), %d key heads",
+                     i, sp.q_rank, sp.kv_rank, sp.rot_dim, sp.rot_dims, sp.rot_base, sp.kv_heads);
+      CREATE_REQUIRE(sp.kv_rank <= 512, "tl_stack_create: layer %d: a key/value latent of %d above 512", i, sp.kv_rank);
+      CREATE_REQUIRE(sp.weights_of == 0, "tl_stack_create: layer %d: a latent layer owns its tensors (it may share a cache: kv_from)", i);
+      L.kv_src = i;
+      if (sp.kv_from > 0) {
+        const int j = sp.kv_from - 1;
+        CREATE_REQUIRE(j < i && st->layers[j].sp.mixer == TL_MIXER_LATENT && st->layers[j].sp.kv_from == 0,
+                       "tl_stack_create: layer %d reads the latent cache of layer %d, which is not an earlier latent layer "
+                       "with a projection of its own", i, j);
+        const tl_layer_spec& o = st->layers[j].sp;
+        CREATE_REQUIRE(o.kv_rank == sp.kv_rank && o.rot_dim == sp.rot_dim && o.rot_dims == sp.rot_dims && o.rot_base == sp.rot_base,
+                       "tl_stack_create: layer %d and layer %d, whose latent cache it reads, differ in latent size or rotation", i, j);
+        L.kv_src = j;
+      }
+      const bool own_kv = L.kv_src == i;
+      const int qh = sp.dim + sp.rot_dim, ah = sp.kv_rank + sp.rot_dim;
+      L.qd = sp.heads * qh;
+      L.kd = own_kv ? sp.kv_rank + sp.rot_dim : 0;
+      L.vd = 0;
+      L.od = sp.heads * sp.vdim;
+      L.gate_off = sp.q_rank + L.kd;
+      L.pd = L.gate_off + (sp.head_gate ? sp.heads : 0);
+      if (own_kv) st->cache_bytes += sizeof(float) * (size_t)cfg->max_positions * L.kd;
+      st->max_lq = L.qd > st->max_lq ? L.qd : st->max_lq;
+      st->max_lqa = sp.heads * ah > st->max_lqa ? sp.heads * ah : st->max_lqa;
+      st->max_od = sp.heads * sp.kv_rank > st->max_od ? sp.heads * sp.kv_rank : st->max_od;  // the weighted latents of all heads
+      L.expect.insert({"mix.dq", "mix.dq.norm", "mix.uq", "mix.uk", "mix.uv", "mix.o"});
+      if (own_kv) L.expect.insert({"mix.dkv", "mix.dkv.norm"});
+      if (sp.head_gate) L.expect.insert("mix.g");
+      if ((rc = dev_alloc(st, &L.wuq, (size_t)L.qd * sp.q_rank))) break;
+      if ((rc = dev_alloc(st, &L.wukt, (size_t)sp.heads * sp.kv_rank * sp.dim))) break;
+      if ((rc = dev_alloc(st, &L.wuv, (size_t)sp.heads * sp.vdim * sp.kv_rank))) break;
+      if ((rc = dev_alloc(st, &L.dq_norm, sp.q_rank))) break;
+      if ((rc = dev_alloc(st, &L.dkv_norm, sp.kv_rank))) break;
+      if (sp.rot_dims > 0) {
+        std::vector<double> f(sp.rot_dims / 2);
+        float unused = 1.0f;
+        tl_rotary_frequencies(sp.rot_dims, sp.rot_base, 0.0, 0.0, 0.0, 0.0, f.data(), &unused);
+        if ((rc = dev_alloc(st, &L.freq, f.size()))) break;
+        if (hipMemcpy(L.freq, f.data(), sizeof(double) * f.size(), hipMemcpyHostToDevice) != hipSuccess) {
+          tl_set_error("tl_stack_create: upload of the rotary frequencies failed");
+          return fail(1);
+        }
+      }
+    } else if (sp.mixer == TL_MIXER_GDELTA) {
+      CREATE_REQUIRE(sp.decay_rank > 0 && sp.vdim == sp.dim && sp.kv_heads == sp.heads && sp.dim <= 256,
+                     "tl_stack_create: layer %d: generalized delta rule with inner size %d, head sizes %d / %d (equal, at most 256), "
+                     "%d key heads", i, sp.decay_rank, sp.dim, sp.vdim, sp.kv_heads);
+      CREATE_REQUIRE(sp.weights_of == 0, "tl_stack_create: layer %d: a generalized delta layer owns its tensors", i);
+      const int hd = sp.heads * sp.dim;
+      L.qd = L.kd = L.vd = L.od = hd;
+      L.pd = 5 * hd + sp.decay_rank;
+      st->max_gd = hd > st->max_gd ? hd : st->max_gd;
+      ++st->gdelta_layers;
+      st->cache_bytes += sizeof(float) * (size_t)sp.heads * sp.dim * sp.dim;
+      L.expect.insert({"mix.r", "mix.k", "mix.v", "mix.g", "mix.a", "mix.a.b", "mix.w1", "mix.w2", "mix.w0", "mix.norm", "mix.o"});
+      if ((rc = dev_alloc(st, &L.wa2, (size_t)hd * sp.decay_rank))) break;
+      if ((rc = dev_alloc(st, &L.w0, hd))) break;
+      if ((rc = dev_alloc(st, &L.a_bias, hd))) break;
+      if ((rc = dev_alloc(st, &L.onorm, hd))) break;
     } else {
-      CREATE_REQUIRE(sp.block == TL_BLOCK_PARALLEL, "tl_stack_create: layer %d: the delta rule runs in parallel blocks only", i);
       CREATE_REQUIRE(sp.conv_taps >= 1 && sp.conv_taps <= 64 && sp.decay_rank > 0 && sp.gate_rank > 0,
                      "tl_stack_create: layer %d: %d taps, inner sizes %d / %d", i, sp.conv_taps, sp.decay_rank, sp.gate_rank);
       CREATE_REQUIRE(sp.dim <= 256 && sp.vdim <= 512, "tl_stack_create: layer %d: key size %d above 256 or value size %d above 512", i,
@@ -277,6 +378,11 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
       if ((rc = dev_alloc(st, &L.norm1, W))) break;
       if ((rc = dev_alloc(st, &L.norm2, W))) break;
       L.expect.insert("norm1");
+      if (lnorm) {
+        if ((rc = dev_alloc(st, &L.norm1_b, W))) break;
+        if ((rc = dev_alloc(st, &L.norm2_b, W))) break;
+        L.expect.insert("norm1.b");
+      }
       if (dyt) {
         if ((rc = dev_alloc(st, &L.norm1_b, W))) break;
         if ((rc = dev_alloc(st, &L.norm1_alpha, 1))) break;
@@ -326,8 +432,19 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
         if ((rc = dev_alloc(st, &L.sdown, W * sp.shared_ff))) break;
       }
       st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
+    } else if (sp.mlp == TL_MLP_UNIT) {
+      CREATE_REQUIRE(sp.shared_ff > 0 && sp.act >= TL_ACT_NONE && sp.act <= TL_ACT_TANH,
+                     "tl_stack_create: layer %d: a feed-forward of size %d with activation kind %d", i, sp.shared_ff, sp.act);
+      if (own) {
+        L.expect.insert({"norm2", "norm2.b", "mlp.up", "mlp.down"});
+        if (sp.act == TL_ACT_XIELU) L.expect.insert("mlp.act");
+        if ((rc = dev_alloc(st, &L.sgu, (size_t)sp.shared_ff * W))) break;
+        if ((rc = dev_alloc(st, &L.sdown, W * sp.shared_ff))) break;
+      }
+      st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
     } else if (own) {
       L.optional.insert("norm2");
+      if (lnorm) L.optional.insert("norm2.b");
     }
     st->max_qkv = L.pd > st->max_qkv ? L.pd : st->max_qkv;
     st->max_od = L.od > st->max_od ? L.od : st->max_od;
@@ -338,9 +455,11 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
   if (rc) return fail(rc);
   if ((rc = dev_alloc(st, &st->embed, (size_t)cfg->vocab * W)) || (rc = dev_alloc(st, &st->head, (size_t)cfg->vocab * W)) ||
       (rc = dev_alloc(st, &st->embed_norm, W)) || (rc = dev_alloc(st, &st->final_norm, W)) ||
-      (rc = dev_alloc(st, &st->final_b, W)) || (rc = dev_alloc(st, &st->final_alpha, 1)))
+      (rc = dev_alloc(st, &st->final_b, W)) || (rc = dev_alloc(st, &st->final_alpha, 1)) ||
+      (rc = dev_alloc(st, &st->embed_norm_b, W)))
     return fail(rc);
-  st->need_globals = 1 | 2 | 8 | (cfg->embed_norm ? 4 : 0) | (cfg->norm == TL_NORM_DYT ? 16 | 32 : 0);
+  st->need_globals = 1 | 2 | 8 | (cfg->embed_norm ? 4 : 0) | (cfg->norm == TL_NORM_DYT ? 16 | 32 : 0) |
+                     (cfg->norm == TL_NORM_LAYER ? 16 | (cfg->embed_norm ? 64 : 0) : 0);
   if (const char* e = getenv("TL_STACK_CHUNK")) st->chunk = atoi(e) > 0 ? atoi(e) : st->chunk;
   if (const char* e = getenv("TL_STACK_GEMV")) st->gemv_decode = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FUSE_ROUTER")) st->fuse_router = atoi(e) != 0;
@@ -389,6 +508,7 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
   if (n == "embed") { st->got_globals |= 1; MATRIX(st->embed, V, W); }
   if (n == "head") { st->got_globals |= 2; MATRIX(st->head, V, W); }
   if (n == "embed.norm") { st->got_globals |= 4; VECTOR(st->embed_norm, W); }
+  if (n == "embed.norm.b") { st->got_globals |= 64; VECTOR(st->embed_norm_b, W); }
   if (n == "final.norm") { st->got_globals |= 8; VECTOR(st->final_norm, W); }
   if (n == "final.norm.b") { st->got_globals |= 16; VECTOR(st->final_b, W); }
   if (n == "final.norm.alpha") { st->got_globals |= 32; VECTOR(st->final_alpha, 1); }
@@ -407,6 +527,64 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
   if (r == "norm1.b") VECTOR(L.norm1_b, W);
   if (r == "norm1.alpha") VECTOR(L.norm1_alpha, 1);
   if (r == "norm2") VECTOR(L.norm2, W);
+  if (r == "norm2.b") VECTOR(L.norm2_b, W);
+  if (sp.mixer == TL_MIXER_LATENT) {
+    const long long qh = sp.dim + sp.rot_dim;
+    if (r == "mix.dq") MATRIX(L.wqkv, sp.q_rank, W);
+    if (r == "mix.dkv") MATRIX(L.wqkv + (size_t)sp.q_rank * W, L.kd, W);
+    if (r == "mix.g") MATRIX(L.wqkv + (size_t)L.gate_off * W, sp.heads, W);
+    if (r == "mix.dq.norm") VECTOR(L.dq_norm, sp.q_rank);
+    if (r == "mix.dkv.norm") VECTOR(L.dkv_norm, sp.kv_rank);
+    if (r == "mix.uq") MATRIX(L.wuq, sp.heads * qh, sp.q_rank);
+    if (r == "mix.uv") MATRIX(L.wuv, (long long)sp.heads * sp.vdim, sp.kv_rank);
+    if (r == "mix.o") MATRIX(L.wo, W, L.od);
+    if (r == "mix.uk") {  // [heads * dim][kv_rank] -> per head its transpose [kv_rank][dim]
+      TL_REQUIRE(type == TL_BF16 && shape_is(shape, ndim, (long long)sp.heads * sp.dim, sp.kv_rank),
+                 "tl_stack_set_tensor: %s is not a bf16 matrix of %lld x %d", name, (long long)sp.heads * sp.dim, sp.kv_rank);
+      const uint16_t* src = static_cast<const uint16_t*>(host);
+      std::vector<uint16_t> tr((size_t)sp.heads * sp.kv_rank * sp.dim);
+      for (int hh = 0; hh < sp.heads; ++hh)
+        for (int d = 0; d < sp.dim; ++d)
+          for (int c = 0; c < sp.kv_rank; ++c)
+            tr[((size_t)hh * sp.kv_rank + c) * sp.dim + d] = src[((size_t)hh * sp.dim + d) * sp.kv_rank + c];
+      return upload_bf16(L.wukt, tr.data(), tr.size(), s);
+    }
+  }
+  if (sp.mixer == TL_MIXER_GDELTA) {
+    const long long hd = (long long)sp.heads * sp.dim;
+    if (r == "mix.r") MATRIX(L.wqkv, hd, W);
+    if (r == "mix.k") MATRIX(L.wqkv + (size_t)hd * W, hd, W);
+    if (r == "mix.v") MATRIX(L.wqkv + (size_t)2 * hd * W, hd, W);
+    if (r == "mix.g") MATRIX(L.wqkv + (size_t)3 * hd * W, hd, W);
+    if (r == "mix.a") MATRIX(L.wqkv + (size_t)4 * hd * W, hd, W);
+    if (r == "mix.w1") MATRIX(L.wqkv + (size_t)5 * hd * W, sp.decay_rank, W);
+    if (r == "mix.w2") MATRIX(L.wa2, hd, sp.decay_rank);
+    if (r == "mix.w0") VECTOR(L.w0, hd);
+    if (r == "mix.a.b") VECTOR(L.a_bias, hd);
+    if (r == "mix.norm") VECTOR(L.onorm, hd);
+    if (r == "mix.o") MATRIX(L.wo, W, L.od);
+  }
+  if (sp.mlp == TL_MLP_UNIT) {
+    const long long ff = sp.shared_ff;
+    if (r == "mlp.up") MATRIX(L.sgu, ff, W);
+    if (r == "mlp.down") MATRIX(L.sdown, W, ff);
+    if (r == "mlp.act") {  // two numbers (p, q): P = softplus(p), Q = 1/2 + softplus(q), formed once, in double
+      TL_REQUIRE(shape_is(shape, ndim, 2), "tl_stack_set_tensor: %s does not have 2 elements", name);
+      float pq[2];
+      if (type == TL_BF16) {
+        for (int j = 0; j < 2; ++j) {
+          const uint32_t bits = (uint32_t) static_cast<const uint16_t*>(host)[j] << 16;
+          memcpy(&pq[j], &bits, 4);
+        }
+      } else {
+        memcpy(pq, host, 8);
+      }
+      auto softplus = [](double z) { return z > 30.0 ? z : log1p(exp(z)); };
+      L.act_p = (float)softplus(pq[0]);
+      L.act_q = (float)(0.5 + softplus(pq[1]));
+      return 0;
+    }
+  }
   if (r == "mix.q") MATRIX(L.wqkv, L.qd, W);
   if (r == "mix.k") MATRIX(L.wqkv + (size_t)L.qd * W, L.kd, W);
   if (r == "mix.v") MATRIX(L.wqkv + (size_t)(L.qd + L.kd) * W, L.vd, W);
@@ -482,6 +660,16 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
       p += (size_t)st->cfg.max_positions * L.kd;
       L.vc = p;
       p += (size_t)st->cfg.max_positions * L.vd;
+    } else if (L.sp.mixer == TL_MIXER_LATENT) {
+      if (L.kd) {
+        L.ckv = p;
+        p += (size_t)st->cfg.max_positions * L.kd;
+      } else {
+        L.ckv = st->layers[L.kv_src].ckv;  // an earlier layer: already placed
+      }
+    } else if (L.sp.mixer == TL_MIXER_GDELTA) {
+      L.state = p;
+      p += (size_t)L.sp.heads * L.sp.dim * L.sp.dim;
     } else {
       L.state = p;
       p += (size_t)L.sp.heads * L.sp.vdim * L.sp.dim;
@@ -498,18 +686,33 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
   TL_TRY(dev_alloc(st, &st->xn, C * W));
   if (st->max_dc) {
     TL_TRY(dev_alloc(st, &st->dq, C * st->max_dc));
-    TL_TRY(dev_alloc(st, &st->da, C * st->max_da));
+    if (st->max_da > st->max_gd) st->max_gd = st->max_da;  // one buffer serves both recurrences' decay pre-activations
     TL_TRY(dev_alloc(st, &st->ddecay, C * st->max_da));
     TL_TRY(dev_alloc(st, &st->dg, C * st->max_od));
     TL_TRY(dev_alloc(st, &st->dbeta, C * st->max_heads));
+  }
+  if (st->max_lq) {
+    TL_TRY(dev_alloc(st, &st->lq, C * st->max_lq));
+    TL_TRY(dev_alloc(st, &st->lqa, C * st->max_lqa));
+  }
+  if (st->max_gd) {
+    TL_TRY(dev_alloc(st, &st->da, C * st->max_gd));
+  }
+  if (st->gdelta_layers) {
+    TL_TRY(dev_alloc(st, &st->gw, C * st->max_gd));
+    TL_TRY(dev_alloc(st, &st->gu, C * st->max_gd));
+    TL_TRY(dev_alloc(st, &st->gau, C * st->max_gd));
+    TL_TRY(dev_alloc(st, &st->grau, C * st->max_heads));
+    TL_TRY(dev_alloc(st, &st->grk, C * st->max_heads));
   }
   {
     size_t ws = 1;
     for (const Layer& L : st->layers)
       for (int T = 1; T <= 4; ++T) {
-        if (L.sp.mixer != TL_MIXER_SWA) continue;
-        const size_t n = tl_swa_ws_floats(T, L.sp.heads, L.sp.vdim,
-                                          tl_swa_splits(T, L.sp.window, st->cfg.max_positions, L.sp.keep_first));
+        if (L.sp.mixer != TL_MIXER_SWA && L.sp.mixer != TL_MIXER_LATENT) continue;
+        const bool lat = L.sp.mixer == TL_MIXER_LATENT;
+        const size_t n = tl_swa_ws_floats(T, L.sp.heads, lat ? L.sp.kv_rank : L.sp.vdim,
+                                          tl_swa_splits(T, lat ? 0 : L.sp.window, st->cfg.max_positions, lat ? 0 : L.sp.keep_first));
         ws = n > ws ? n : ws;
       }
     TL_TRY(dev_alloc(st, &st->swa_ws, ws));
@@ -571,7 +774,9 @@ int tl_stack_cache_ptr(TlStack* st, int which, int layer, void** out) {
   TL_REQUIRE(layer >= 0 && layer < (int)st->layers.size(), "tl_stack_cache_ptr: layer %d out of range", layer);
   const Layer& L = st->layers[layer];
   // attention: 0 keys, 1 values; delta rule: 0 the state S [heads][vdim][dim], 1 the convolution's history
+  // latent attention: 0 the rows [max_pos][kv_rank + rot_dim] this layer reads; generalized delta rule: 0 the state
   if (L.sp.mixer == TL_MIXER_SWA) *out = which == 0 ? L.kc : L.vc;
+  else if (L.sp.mixer == TL_MIXER_LATENT) *out = L.ckv;
   else *out = which == 0 ? L.state : L.hist;
   return 0;
 }
@@ -582,6 +787,17 @@ void tl_stack_bytes_per_token(const TlStack* st, int pos, double* weight_bytes, 
   for (const Layer& L : st->layers) {
     const tl_layer_spec& sp = L.sp;
     wb += 2.0 * W * (L.pd + L.od);
+    if (sp.mlp == TL_MLP_UNIT) wb += 2.0 * W * 2.0 * sp.shared_ff;
+    if (sp.mixer == TL_MIXER_LATENT) {
+      wb += 2.0 * ((double)L.qd * sp.q_rank + (double)sp.heads * sp.kv_rank * (sp.dim + sp.vdim));
+      kb += 4.0 * (pos + 2.0) * (sp.kv_rank + sp.rot_dim);  // every head reads the same rows: counted once
+      continue;
+    }
+    if (sp.mixer == TL_MIXER_GDELTA) {
+      wb += 2.0 * (double)sp.heads * sp.dim * sp.decay_rank;
+      kb += 2.0 * 4.0 * sp.heads * sp.dim * sp.dim;
+      continue;
+    }
     if (sp.mlp == TL_MLP_MOE)
       wb += 2.0 * W * (sp.experts + 3.0 * sp.expert_ff * sp.top + 3.0 * sp.shared_ff + (sp.shared_gate ? 1.0 : 0.0));
     if (sp.mlp == TL_MLP_DENSE) wb += 2.0 * W * 3.0 * sp.shared_ff;
@@ -804,6 +1020,8 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
     q.vmix = L.vmix_mode;
     q.v_first = st->v_first;
     q.lambda = Wt.lambda;
+    q.q_temp_coef = sp.q_temp_coef;
+    q.q_temp_every = sp.q_temp_every;
     TL_TRY(tl_launch_qkv_post(q, s));
   }
   SwaArgs a = {};
@@ -823,6 +1041,7 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
   a.pos_dev = pos_dev;
   a.keep_first = sp.keep_first;
   a.sigmoid = sp.attn_weight == TL_ATTN_SIGMOID;
+  a.sink = sp.attn_weight == TL_ATTN_SOFTMAX_SINK;
   a.head_bias = a.sigmoid ? Wt.pb : nullptr;
   a.nsplit = tl_swa_splits(T, sp.window, c.max_positions, sp.keep_first);
   a.ws = st->swa_ws;
@@ -874,6 +1093,176 @@ int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, 
   TL_TRY(tl_launch_delta_scan(d, s));
   TL_TRY(tl_launch_gated_head_norm(st->att, st->dg, Wt.onorm, T, sp.heads, sp.vdim, st->cfg.norm_eps, s));
   return project(st, Wt.wo, W, L.od, st->att, L.od, st->proj, W, T, s);
+}
+
+// one product per head: y[t][n * y_stride ..] = W[n] x[t][n * x_stride ..]
+int project_heads(TlStack* st, const uint16_t* w, int heads, int rows, int cols, const float* x, int ldx, int x_stride, float* y,
+                  int ldy, int y_stride, int T, hipStream_t s) {
+  if (T == 1 && st->gemv_decode) return tl_launch_dense_gemv_heads(w, heads, rows, cols, x, x_stride, y, y_stride, s);
+  DenseArgs d = {};
+  d.w = w;
+  d.rows = rows;
+  d.cols = cols;
+  d.x = x;
+  d.ldx = ldx;
+  d.y = y;
+  d.ldy = ldy;
+  d.T = T;
+  d.terms = terms_for(st, T);
+  d.groups = heads;
+  d.x_gstride = x_stride;
+  d.y_gstride = y_stride;
+  return tl_launch_dense_gemm(d, s);
+}
+
+// y = act(W x) on the rows from act_from on
+int project_act(TlStack* st, const uint16_t* w, int rows, int cols, const float* x, int ldx, float* y, int ldy, int T, int act,
+                int act_from, float act_p, float act_q, hipStream_t s) {
+  if (T == 1 && st->gemv_decode) return tl_launch_dense_gemv_act(w, rows, cols, x, y, GemvActArgs{act, act_from, act_p, act_q}, s);
+  DenseArgs d = {};
+  d.w = w;
+  d.rows = rows;
+  d.cols = cols;
+  d.x = x;
+  d.ldx = ldx;
+  d.y = y;
+  d.ldy = ldy;
+  d.T = T;
+  d.terms = terms_for(st, T);
+  d.act = act;
+  d.act_from = act_from;
+  d.act_p = act_p;
+  d.act_q = act_q;
+  return tl_launch_dense_gemm(d, s);
+}
+
+int latent_mixer(TlStack* st, Layer& L, const float* in, int T, int start_pos, const int* pos_dev, hipStream_t s) {
+  const tl_layer_spec& sp = L.sp;
+  const tl_stack_config& c = st->cfg;
+  const int W = c.width, ld = L.pd, H = sp.heads, qh = sp.dim + sp.rot_dim, ah = sp.kv_rank + sp.rot_dim;
+  TL_TRY(project(st, L.wqkv, ld, W, in, W, st->qkv, ld, T, s));  // query latent | (key/value latent | rotated part) | gates
+  LatentPostArgs p = {};
+  p.p = st->qkv;
+  p.ld = ld;
+  p.q_rank = sp.q_rank;
+  p.kv_rank = sp.kv_rank;
+  p.rot_dim = sp.rot_dim;
+  p.q_norm = L.dq_norm;
+  p.kv_norm = L.kd ? L.dkv_norm : nullptr;
+  p.eps = c.norm_eps;
+  p.rot_dims = sp.rot_dims;
+  p.freq = L.freq;
+  p.cache = L.kd ? L.ckv : nullptr;
+  p.T = T;
+  p.start_pos = start_pos;
+  p.pos_dev = pos_dev;
+  TL_TRY(tl_launch_latent_post(p, s));
+  TL_TRY(project(st, L.wuq, L.qd, sp.q_rank, st->qkv, ld, st->lq, L.qd, T, s));
+  // the plain part of head n's query through W_uk,n^T: scores against the cached latent itself
+  TL_TRY(project_heads(st, L.wukt, H, sp.kv_rank, sp.dim, st->lq, L.qd, qh, st->lqa, H * ah, ah, T, s));
+  LatentQueryArgs q = {};
+  q.q = st->lq;
+  q.qa = st->lqa;
+  q.heads = H;
+  q.dim = sp.dim;
+  q.rot_dim = sp.rot_dim;
+  q.kv_rank = sp.kv_rank;
+  q.rot_dims = sp.rot_dims;
+  q.freq = L.freq;
+  q.T = T;
+  q.start_pos = start_pos;
+  q.pos_dev = pos_dev;
+  TL_TRY(tl_launch_latent_query(q, s));
+  SwaArgs a = {};
+  a.q = st->lqa;
+  a.ldq = H * ah;
+  a.kc = L.ckv;  // keys: the whole row; values: its first kv_rank columns
+  a.vc = L.ckv;
+  a.kld = ah;
+  a.vld = ah;
+  a.out = st->att;
+  a.T = T;
+  a.heads = H;
+  a.kv_heads = 1;
+  a.dim = ah;
+  a.vdim = sp.kv_rank;
+  a.scale = sp.scale;
+  a.start_pos = start_pos;
+  a.pos_dev = pos_dev;
+  a.nsplit = tl_swa_splits(T, 0, c.max_positions, 0);
+  a.ws = st->swa_ws;
+  a.done_cnt = st->swa_cnt;
+  TL_TRY(tl_launch_swa(a, s));
+  // head n's weighted latent through W_uv,n (lq is free again)
+  TL_TRY(project_heads(st, L.wuv, H, sp.vdim, sp.kv_rank, st->att, H * sp.kv_rank, sp.kv_rank, st->lq, L.od, sp.vdim, T, s));
+  if (sp.head_gate) TL_TRY(tl_launch_head_gate(st->lq, st->qkv + L.gate_off, ld, T, H, sp.vdim, s));
+  return project(st, L.wo, W, L.od, st->lq, L.od, st->proj, W, T, s);
+}
+
+int gdelta_mixer(TlStack* st, Layer& L, const float* in, int T, hipStream_t s) {
+  const tl_layer_spec& sp = L.sp;
+  const int W = st->cfg.width, ld = L.pd, hd = sp.heads * sp.dim;
+  // r | k | v | gate | a | tanh(w1 h)
+  TL_TRY(project_act(st, L.wqkv, ld, W, in, W, st->qkv, ld, T, TL_ACT_TANH, 5 * hd, 0.0f, 0.0f, s));
+  TL_TRY(project(st, L.wa2, hd, sp.decay_rank, st->qkv + 5 * hd, ld, st->da, hd, T, s));
+  GDeltaPreArgs p = {};
+  p.p = st->qkv;
+  p.ld = ld;
+  p.dw = st->da;
+  p.w0 = L.w0;
+  p.a_bias = L.a_bias;
+  p.decay_scale = sp.decay_scale;
+  p.T = T;
+  p.heads = sp.heads;
+  p.dim = sp.dim;
+  p.w = st->gw;
+  p.u = st->gu;
+  p.au = st->gau;
+  p.rau = st->grau;
+  p.rk = st->grk;
+  TL_TRY(tl_launch_gdelta_pre(p, s));
+  GDeltaScanArgs d = {};
+  d.r = st->qkv;
+  d.k = st->qkv + hd;
+  d.v = st->qkv + 2 * hd;
+  d.ld = ld;
+  d.w = st->gw;
+  d.u = st->gu;
+  d.au = st->gau;
+  d.rau = st->grau;
+  d.rk = st->grk;
+  d.state = L.state;
+  d.o = st->att;
+  d.T = T;
+  d.heads = sp.heads;
+  d.dim = sp.dim;
+  d.vdim = sp.dim;
+  TL_TRY(tl_launch_gdelta_scan(d, s));
+  TL_TRY(tl_launch_gated_head_norm_rows(st->att, st->qkv + 3 * hd, ld, L.onorm, 1, T, sp.heads, sp.dim, st->cfg.norm_eps, s));
+  return project(st, L.wo, W, L.od, st->att, L.od, st->proj, W, T, s);
+}
+
+LnParams ln1_of_layer(const Layer& Wt) { return LnParams{Wt.norm1, Wt.norm1_b}; }
+
+// h = norm1(x) is already in st->h. x += mixer(h); then, with a feed-forward, h = norm2(x), x += ff(h). The launch that
+// finishes x writes the norm of the next layer's first sublayer into st->h.
+int pre_norm_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_dev, hipStream_t s) {
+  Layer& L = st->layers[li];
+  const Layer& Wt = st->layers[L.wsrc];
+  const tl_layer_spec& sp = L.sp;
+  const tl_stack_config& c = st->cfg;
+  const int W = c.width;
+  if (sp.mixer == TL_MIXER_SWA) TL_TRY(swa_mixer(st, L, Wt, st->h, T, start_pos, pos_dev, s));
+  else if (sp.mixer == TL_MIXER_LATENT) TL_TRY(latent_mixer(st, L, st->h, T, start_pos, pos_dev, s));
+  else TL_TRY(gdelta_mixer(st, L, st->h, T, s));
+  LnParams next = {};
+  if (li + 1 < st->layers.size()) next = ln1_of_layer(st->layers[st->layers[li + 1].wsrc]);
+  if (sp.mlp == TL_MLP_NONE) return tl_launch_resid_ln(st->x, st->proj, T, W, next, c.norm_eps, st->h, s);
+  TL_TRY(tl_launch_resid_ln(st->x, st->proj, T, W, LnParams{Wt.norm2, Wt.norm2_b}, c.norm_eps, st->h, s));
+  const int ff = sp.shared_ff;
+  TL_TRY(project_act(st, Wt.sgu, ff, W, st->h, W, st->sact, ff, T, sp.act, 0, Wt.act_p, Wt.act_q, s));
+  TL_TRY(project(st, Wt.sdown, W, ff, st->sact, ff, st->sout, W, T, s));
+  return tl_launch_resid_ln(st->x, st->sout, T, W, next, c.norm_eps, st->h, s);
 }
 
 DytParams dyt_of_layer(const Layer& Wt) { return DytParams{Wt.norm1_alpha, Wt.norm1, Wt.norm1_b}; }
@@ -967,8 +1356,12 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
   TL_REQUIRE(n_rows >= 0 && n_rows <= T && (n_rows == 0 || logits_dev), "tl_stack_forward: bad logits request");
   const tl_stack_config& c = st->cfg;
   const int W = c.width;
-  const bool dyt = c.norm == TL_NORM_DYT;
-  if (c.embed_norm) {
+  const bool dyt = c.norm == TL_NORM_DYT, lnorm = c.norm == TL_NORM_LAYER;
+  if (lnorm) {
+    const LnParams emb = c.embed_norm ? LnParams{st->embed_norm, st->embed_norm_b} : LnParams{};
+    TL_TRY(tl_launch_embed_ln(st->embed, c.vocab, W, tokens_dev, T, emb, ln1_of_layer(st->layers[st->layers[0].wsrc]), c.norm_eps,
+                              st->x, st->h, s));
+  } else if (c.embed_norm) {
     TL_TRY(tl_launch_embed_norm(st->embed, c.vocab, W, tokens_dev, T, st->embed_norm, c.norm_eps, st->x, s));
     if (dyt) TL_TRY(tl_launch_dyt_rows(st->x, W, nullptr, T, dyt_of_layer(st->layers[st->layers[0].wsrc]), st->h, s));
   } else {
@@ -980,6 +1373,8 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
     const tl_layer_spec& sp = L.sp;
     if (sp.block == TL_BLOCK_PARALLEL) {
       TL_TRY(parallel_layer(st, li, T, start_pos, pos_dev, s));
+    } else if (sp.block == TL_BLOCK_PRE_NORM) {
+      TL_TRY(pre_norm_layer(st, li, T, start_pos, pos_dev, s));
     } else {
       const Layer& Wt = st->layers[L.wsrc];
       TL_TRY(swa_mixer(st, L, Wt, st->x, T, start_pos, pos_dev, s));
@@ -1012,6 +1407,7 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
     if (!rows_dev && n_rows == 1) src = st->x + (size_t)last * W;
     TL_REQUIRE(rows_dev || n_rows == 1 || n_rows == T, "tl_stack_forward: %d rows without a list", n_rows);
     if (dyt) TL_TRY(tl_launch_dyt_rows(src, W, rows_dev, n_rows, DytParams{st->final_alpha, st->final_norm, st->final_b}, st->xn, s));
+    else if (lnorm) TL_TRY(tl_launch_ln_rows(src, W, rows_dev, n_rows, LnParams{st->final_norm, st->final_b}, c.norm_eps, st->xn, s));
     else TL_TRY(tl_launch_norm_rows(src, W, rows_dev, n_rows, st->final_norm, c.norm_eps, st->xn, s));
     TL_TRY(project(st, st->head, c.vocab, W, st->xn, W, logits_dev, c.vocab, n_rows, s, c.logit_softcap));
   }

@@ -3,6 +3,9 @@
 // j < keep_first as well (the first tokens of the sequence stay visible at their true positions); the weights are an ordinary
 // softmax or, in sigmoid mode, sigmoid(score + bias[head]) without normalisation over the keys. Everything in FP32. Key size
 // (dim) and value size (vdim) are independent; query head h reads key/value head h / (heads / kv_heads).
+// With a sink the softmax's denominator has one more term exp(0): where partial (max, sum) pairs are merged, the maximum is
+// taken together with 0 and exp(-max) joins the sum once. The rows of the caches may be further apart than a row is wide
+// (kld, vld): a cache of latent rows is read as keys over its whole row and as values over its first vdim columns.
 // Sigmoid mode runs through the softmax machinery with the running maximum pinned to 0: every correction factor is exp(0) = 1,
 // the partial sums of waves and splits are simply added, and the final division falls away.
 //
@@ -38,8 +41,9 @@ __device__ __forceinline__ void swa_merge_records(const SwaArgs& a, int t, int h
   float M = mz;
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  if (a.sink) M = fmaxf(M, 0.0f);
   const float fz = mz == -INFINITY ? 0.0f : expf(mz - M);
-  float L = 0.0f;
+  float L = a.sink ? expf(-M) : 0.0f;
   for (int z = 0; z < a.nsplit; ++z) L += __shfl(lz * fz, z);  // in split order
   float* op = a.out + (size_t)t * a.heads * a.vdim + (size_t)h * a.vdim;
   for (int d0 = 0; d0 < a.vdim; d0 += 64) {  // every lane stays in the loop: a shuffle reads nothing from a lane that has left
@@ -79,7 +83,7 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   const int nf = a.keep_first > 0 ? (a.keep_first < jlo ? a.keep_first : jlo) : 0;
   const int pf = (nf + 63) >> 6;
   const float hb = a.sigmoid && a.head_bias ? a.head_bias[h] : 0.0f;
-  const int kld = a.kv_heads * a.dim, vld = a.kv_heads * a.vdim;
+  const int kld = a.kld > 0 ? a.kld : a.kv_heads * a.dim, vld = a.vld > 0 ? a.vld : a.kv_heads * a.vdim;
   const float* qp = a.q + (size_t)t * a.ldq + (size_t)h * a.dim;
   for (int d = tid; d < a.dim; d += 256) qs[d] = qp[d];
   __syncthreads();
@@ -183,7 +187,10 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   float M = -INFINITY;
 #pragma unroll
   for (int w = 0; w < SWA_WAVES; ++w) M = fmaxf(M, ml[w * 2]);
-  float f[SWA_WAVES], L = 0.0f;
+  // the sink joins where the LAST merge happens: here without splits, in swa_merge_records with them
+  const bool sink_here = a.sink && nsplit == 1;
+  if (sink_here) M = fmaxf(M, 0.0f);
+  float f[SWA_WAVES], L = sink_here ? expf(-M) : 0.0f;
 #pragma unroll
   for (int w = 0; w < SWA_WAVES; ++w) {
     f[w] = ml[w * 2] == -INFINITY ? 0.0f : expf(ml[w * 2] - M);  // a wave without a piece counts nothing
@@ -268,7 +275,7 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   const int head = blockIdx.y, q0 = blockIdx.x * 32;
   const int g = head / (a.heads / a.kv_heads);
   const int start = a.pos_dev ? *a.pos_dev : a.start_pos;
-  const int kld = a.kv_heads * a.dim, vld = a.kv_heads * a.vdim;
+  const int kld = a.kld > 0 ? a.kld : a.kv_heads * a.dim, vld = a.vld > 0 ? a.vld : a.kv_heads * a.vdim;
   const int last_i = q0 + 31 < a.T ? q0 + 31 : a.T - 1;
   const int qpos = start + (q0 + r < a.T ? q0 + r : a.T - 1);  // rows beyond the chunk repeat its last query; never stored
   const int last_q = start + last_i;
@@ -282,8 +289,8 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   const float hb = a.sigmoid && a.head_bias ? a.head_bias[head] : 0.0f;
   // a row that no query of the tile can see (it carries weight 0) is read from a row that one of them can
   auto clamp_row = [&](int pr) { return pr > last_q ? last_q : (pr < klo && pr >= a.keep_first) ? klo : pr; };
-  const bool kvec = (a.dim & 3) == 0 && ((size_t)a.kc & 15) == 0;
-  const bool vvec = (a.vdim % DB) == 0 && (DB == 1 || (((size_t)a.vc & 15) == 0 && (DB != 3)));
+  const bool kvec = (a.dim & 3) == 0 && (kld & 3) == 0 && ((size_t)a.kc & 15) == 0;
+  const bool vvec = (a.vdim % DB) == 0 && (DB == 1 || (((size_t)a.vc & 15) == 0 && (DB != 3) && (vld % DB) == 0));
   // piece i (d = 8 i + 4 h + 0..3) of the lane's key row of a tile; rows outside [klo, last_q] are seen by no query of the
   // tile (masked below): their loads stay inside that range, so that nothing is read that the tile could not read
   auto load_k4 = [&](int tile, int i) -> swa_f32x4 {
@@ -421,10 +428,11 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
     float M = -INFINITY;
 #pragma unroll
     for (int w = 0; w < SWA_WAVES; ++w) M = fmaxf(M, sm_m[w * 32 + r]);  // finite: every query sees itself
+    if (a.sink) M = fmaxf(M, 0.0f);
     const float mw = sm_m[wave * 32 + r];
     sm_f[wave * 32 + r] = mw == -INFINITY ? 0.0f : expf(mw - M);
     if (wave == 0) {
-      float L = 0.0f;
+      float L = a.sink ? expf(-M) : 0.0f;
 #pragma unroll
       for (int w = 0; w < SWA_WAVES; ++w) {
         const float m2 = sm_m[w * 32 + r];
@@ -498,6 +506,9 @@ int tl_launch_swa(const SwaArgs& a, hipStream_t s) {
   TL_REQUIRE(a.pos_dev || a.start_pos >= 0, "swa: negative start position");
   TL_REQUIRE(a.heads <= 65535, "swa: too many heads");
   TL_REQUIRE(a.keep_first >= 0, "swa: negative number of kept first keys");
+  TL_REQUIRE(!a.sink || !a.sigmoid, "swa: a sink belongs to a softmax");
+  TL_REQUIRE((a.kld == 0 || a.kld >= a.kv_heads * a.dim) && (a.vld == 0 || a.vld >= a.kv_heads * a.vdim),
+             "swa: cache rows %d / %d shorter than the heads they hold", a.kld, a.vld);
   if (swa_mfma_wanted(a)) {
     switch ((a.vdim + 31) / 32) {
       case 1: return launch_swa_mfma<1>(a, s);
@@ -574,6 +585,40 @@ extern "C" int tl_window_attention(const float* q_dev, const float* k_cache_dev,
   a.start_pos = start_pos;
   a.keep_first = keep_first;
   a.sigmoid = sigmoid;
+  a.head_bias = head_bias_dev;
+  a.nsplit = tl_swa_splits(num_tokens, window, start_pos + num_tokens, keep_first);
+  if (a.nsplit > 1) {
+    void* ws = nullptr;
+    TL_TRY(tl_scratch(TL_SCRATCH_ATTN, sizeof(float) * tl_swa_ws_floats(num_tokens, heads, vdim, a.nsplit), &ws));
+    a.ws = static_cast<float*>(ws);
+  }
+  return tl_launch_swa(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tl_window_attention_rows(const float* q_dev, const float* k_cache_dev, const float* v_cache_dev, float* out_dev,
+                                        int num_tokens, int start_pos, int heads, int kv_heads, int dim, int vdim, int k_ld,
+                                        int v_ld, int window, int keep_first, float scale, int mode, const float* head_bias_dev,
+                                        void* stream) {
+  TL_REQUIRE(mode >= TL_ATTN_SOFTMAX && mode <= TL_ATTN_SOFTMAX_SINK, "tl_window_attention_rows: weight kind %d", mode);
+  SwaArgs a = {};
+  a.q = q_dev;
+  a.ldq = heads * dim;
+  a.kc = k_cache_dev;
+  a.vc = v_cache_dev;
+  a.out = out_dev;
+  a.T = num_tokens;
+  a.heads = heads;
+  a.kv_heads = kv_heads;
+  a.dim = dim;
+  a.vdim = vdim;
+  a.kld = k_ld;
+  a.vld = v_ld;
+  a.window = window;
+  a.scale = scale;
+  a.start_pos = start_pos;
+  a.keep_first = keep_first;
+  a.sigmoid = mode == TL_ATTN_SIGMOID;
+  a.sink = mode == TL_ATTN_SOFTMAX_SINK;
   a.head_bias = head_bias_dev;
   a.nsplit = tl_swa_splits(num_tokens, window, start_pos + num_tokens, keep_first);
   if (a.nsplit > 1) {

@@ -490,20 +490,53 @@ def _madalorn_spec(sp, i, L, tensors, layers):
             raise ValueError(f"layer {i}: unknown feed-forward kind {ml['kind']!r}")
 
 
+GDELTA_DECAY_SCALE = 0.60653065971263342  # Sogalix: decay = exp(-e^(-1/2) sigmoid(.)), fixed by the design
+
+
+def _sogalix_spec(sp, i, L, tensors):
+    mx, ml = L["mixer"], L.get("mlp")
+    sp.block, sp.heads, sp.dim = 2, mx["heads"], mx["dim"]
+    if L["type"] == "attention":
+        sp.mixer, sp.kv_heads, sp.vdim, sp.scale, sp.attn_weight = 0, mx["kv_heads"], mx["vdim"], float(mx["scale"]), 2
+        qt = mx.get("q_temp")
+        if qt:
+            sp.q_temp_coef, sp.q_temp_every = float(qt["coef"]), int(qt["every"])
+    elif L["type"] == "latent_attention":
+        sp.mixer, sp.kv_heads, sp.vdim, sp.scale = 2, mx["heads"], mx["vdim"], float(mx["scale"])
+        sp.rot_dim, sp.q_rank, sp.kv_rank, sp.head_gate = mx["rot_dim"], mx["q_rank"], mx["kv_rank"], 1
+        rot = mx.get("rot")
+        if rot:
+            sp.rot_dims, sp.rot_base = rot["dims"], float(rot["base"])
+        if mx.get("kv_from") is not None:
+            sp.kv_from = mx["kv_from"] + 1
+    elif L["type"] == "general_delta":
+        sp.mixer, sp.kv_heads, sp.vdim, sp.decay_scale = 3, mx["heads"], mx["dim"], GDELTA_DECAY_SCALE
+        sp.decay_rank = tensors[f"l{i}.mix.w1"].shape[0]
+    else:
+        raise ValueError(f"layer {i}: unknown type {L['type']!r}")
+    if ml is not None:
+        if ml["kind"] != "dense":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {ml['kind']!r}")
+        sp.mlp, sp.act, sp.shared_ff = 3, 1, ml["ff"]
+
+
 def stack_config_struct(config, max_pos, tensors=None):
     """The ctypes form (tl_stack_config) of a layer-list configuration given as config.json's dictionary; returns
     (struct, the array it points into). The C++ host does the same from the file (host/tl_stack_config.cpp); this one
     serves tests and benches that build models in memory. `tensors` gives the inner sizes that only shapes name."""
     layers = config["layers"]
     arr = (capi.LayerSpec * len(layers))()
-    madalorn = config.get("architecture") == "Madalorn"
+    madalorn, sogalix = config.get("architecture") == "Madalorn", config.get("architecture") == "Sogalix"
     for i, L in enumerate(layers):
         if madalorn:
             _madalorn_spec(arr[i], i, L, tensors or {}, layers)
+        elif sogalix:
+            _sogalix_spec(arr[i], i, L, tensors or {})
         else:
             _ralasun_spec(arr[i], i, L)
     c = capi.StackConfig(config["width"], config["vocab"], len(layers), int(max_pos), float(config["norm"]["eps"]), arr,
-                         1 if madalorn else 0, 0 if madalorn else 1, float(config.get("logit_softcap") or 0.0) if madalorn else 0.0)
+                         1 if madalorn else 2 if sogalix else 0, 0 if madalorn else 1,
+                         float(config.get("logit_softcap") or 0.0) if madalorn else 0.0)
     return c, arr
 
 

@@ -17,6 +17,7 @@ const std::vector<ModelFamily>& model_families() {
       {"llama", "gguf", load_llama_gguf},
       {"Ralasun", "folder", load_stack_folder},
       {"Madalorn", "folder", load_stack_folder},
+      {"Sogalix", "folder", load_stack_folder},
   };
   return table;
 }

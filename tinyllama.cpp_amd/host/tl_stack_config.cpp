@@ -17,6 +17,17 @@
 //     "rot": {"base", "dims", "scaling": {"factor", "original", "fast", "slow"}}, "conv"},
 //     "mlp": null | {"kind": "dense", "ff"} | {"kind": "moe", "router": {"experts", "top", "groups": {"count", "keep"}},
 //     "expert": {"ff"}, "shared": null | {"ff"}}}]}
+// Sogalix   pre-norm blocks with layer norms (weight and bias), an embedding norm; three mixers: "attention" = causal softmax
+//           attention over grouped key/value heads with a sink in the denominator and a query temperature that grows with the
+//           logarithm of the position, no rotation; "latent_attention" = queries and keys/values through normalised latents,
+//           one rotated key part shared by the heads, a gate per head, optionally on an earlier layer's cache (kv_from);
+//           "general_delta" = generalized delta rule with decay exp(-e^-1/2 sigmoid(.)) and a removal rate per key channel;
+//           feed-forward W_down act(W_up h) with a two-parameter activation (mlp.act).
+//   {"architecture", "width", "vocab", "norm": {"eps"}, "layers": [{"type": "attention" | "latent_attention" | "general_delta",
+//     "mixer": {"heads", "kv_heads", "dim", "vdim", "scale", "q_temp": {"coef", "every"}} |
+//              {"heads", "dim", "rot_dim", "vdim", "q_rank", "kv_rank", "scale", "rot": {"base", "dims"}, "kv_from": j} |
+//              {"heads", "dim"},
+//     "mlp": null | {"kind": "dense", "ff"}}]}
 #include <chrono>
 #include <cmath>
 #include <fstream>
@@ -32,6 +43,7 @@ namespace tlhost {
 namespace {
 
 constexpr float kGateAlpha = 1.702f;   // Ralasun: g * sigmoid(1.702 g), fixed by the design
+const float kGDeltaDecayScale = 0.60653065971263342f;  // Sogalix: decay = exp(-e^(-1/2) * sigmoid(.)), fixed by the design
 constexpr int kDefaultContext = 4096;  // cache rows when the caller names no context length
 
 void hip_check(int rc, const std::string& what) {
@@ -172,6 +184,63 @@ tl_layer_spec madalorn_layer(const Json& layers, int index, const SafeTensorsFil
   return sp;
 }
 
+tl_layer_spec sogalix_layer(const Json& layers, int index, const SafeTensorsFile& file) {
+  const Json& L = layers.arr[index];
+  const std::string where = "layers[" + std::to_string(index) + "]";
+  tl_layer_spec sp = {};
+  const std::string& type = L.at("type").as_string("type");
+  const Json& mx = L.at("mixer");
+  sp.block = TL_BLOCK_PRE_NORM;
+  sp.heads = geti(mx, "heads");
+  sp.dim = geti(mx, "dim");
+  if (type == "attention") {
+    sp.mixer = TL_MIXER_SWA;
+    sp.kv_heads = geti(mx, "kv_heads");
+    sp.vdim = geti(mx, "vdim");
+    sp.scale = getf(mx, "scale");
+    sp.attn_weight = TL_ATTN_SOFTMAX_SINK;  // the sink is part of the design
+    if (const Json* qt = present(mx, "q_temp")) {
+      sp.q_temp_coef = getf(*qt, "coef");
+      sp.q_temp_every = geti(*qt, "every");
+      if (sp.q_temp_every <= 0) throw std::runtime_error(where + ": q_temp.every must be positive");
+    }
+  } else if (type == "latent_attention") {
+    sp.mixer = TL_MIXER_LATENT;
+    sp.kv_heads = sp.heads;
+    sp.vdim = geti(mx, "vdim");
+    sp.scale = getf(mx, "scale");
+    sp.rot_dim = geti(mx, "rot_dim");
+    sp.q_rank = geti(mx, "q_rank");
+    sp.kv_rank = geti(mx, "kv_rank");
+    sp.head_gate = 1;
+    if (const Json* rot = present(mx, "rot")) {
+      sp.rot_dims = geti(*rot, "dims");
+      sp.rot_base = getf(*rot, "base");
+    }
+    if (const Json* kf = present(mx, "kv_from")) {
+      const int j = (int)kf->as_int("kv_from");
+      if (j < 0 || j >= index) throw std::runtime_error(where + ": kv_from must name an earlier layer");
+      sp.kv_from = j + 1;
+    }
+  } else if (type == "general_delta") {
+    sp.mixer = TL_MIXER_GDELTA;
+    sp.kv_heads = sp.heads;
+    sp.vdim = sp.dim;
+    sp.decay_scale = kGDeltaDecayScale;
+    sp.decay_rank = tensor_rows(file, "l" + std::to_string(index) + ".mix.w1");
+  } else {
+    throw std::runtime_error(where + ": unknown layer type \"" + type + "\"");
+  }
+  if (const Json* ml = present(L, "mlp")) {
+    const std::string& kind = ml->at("kind").as_string("kind");
+    if (kind != "dense") throw std::runtime_error(where + ": unknown feed-forward kind \"" + kind + "\"");
+    sp.mlp = TL_MLP_UNIT;
+    sp.act = TL_ACT_XIELU;
+    sp.shared_ff = geti(*ml, "ff");
+  }
+  return sp;
+}
+
 }  // namespace
 
 void load_stack_folder(const std::string& dir, int device, int max_context, LoadedModel* out) {
@@ -184,12 +253,14 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   const Json& layers = cfg.at("layers");
   if (layers.kind != Json::ARRAY || layers.arr.empty()) throw std::runtime_error("config.json: \"layers\" is empty");
   const std::string arch = cfg.at("architecture").as_string("architecture");
-  const bool madalorn = arch == "Madalorn";
+  const bool madalorn = arch == "Madalorn", sogalix = arch == "Sogalix";
   SafeTensorsFile file;
   file.open(dir + "/model.safetensors");
   std::vector<tl_layer_spec> specs;
   for (size_t i = 0; i < layers.arr.size(); ++i)
-    specs.push_back(madalorn ? madalorn_layer(layers, (int)i, file) : ralasun_layer(layers.arr[i], (int)i, file));
+    specs.push_back(madalorn  ? madalorn_layer(layers, (int)i, file)
+                    : sogalix ? sogalix_layer(layers, (int)i, file)
+                              : ralasun_layer(layers.arr[i], (int)i, file));
   tl_stack_config sc = {};
   sc.width = geti(cfg, "width");
   sc.vocab = geti(cfg, "vocab");
@@ -197,7 +268,7 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   sc.max_positions = max_context > 0 ? max_context : kDefaultContext;
   sc.norm_eps = (float)cfg.at("norm").at("eps").as_double("norm.eps");
   sc.layers = specs.data();
-  sc.norm = madalorn ? TL_NORM_DYT : TL_NORM_RMS_ONE_PLUS;
+  sc.norm = madalorn ? TL_NORM_DYT : sogalix ? TL_NORM_LAYER : TL_NORM_RMS_ONE_PLUS;
   sc.embed_norm = madalorn ? 0 : 1;
   if (madalorn)
     if (const Json* cap = present(cfg, "logit_softcap")) sc.logit_softcap = (float)cap->as_double("logit_softcap");
@@ -212,7 +283,7 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   mc.rms_norm_eps = sc.norm_eps;
   mc.num_attention_heads = specs[0].heads;
   mc.num_key_value_heads = specs[0].kv_heads;
-  mc.intermediate_size = specs[0].mlp == TL_MLP_DENSE ? specs[0].shared_ff : specs[0].expert_ff;
+  mc.intermediate_size = specs[0].mlp == TL_MLP_DENSE || specs[0].mlp == TL_MLP_UNIT ? specs[0].shared_ff : specs[0].expert_ff;
   mc.bos_token_id = -1;  // token ids in, token ids out: such a checkpoint carries no tokenizer
   mc.eos_token_id = -1;
   if (const Json* e = cfg.find("eos"))

@@ -437,6 +437,94 @@ def build_madalorn(config, seed=0, gain=1.0, ranks=(8, 8)):
     return t
 
 
+def sogalix_attention(heads, kv_heads, dim, vdim, q_temp=None, scale=None):
+    """The "mixer" entry of a Sogalix attention layer; q_temp: None or (coef, every)."""
+    mixer = {"dim": dim, "heads": heads, "kv_heads": kv_heads, "vdim": vdim, "scale": float(scale if scale is not None else dim ** -0.5)}
+    if q_temp is not None:
+        mixer["q_temp"] = {"coef": float(q_temp[0]), "every": int(q_temp[1])}
+    return mixer
+
+
+def sogalix_latent(heads, dim, rot_dim, vdim, q_rank, kv_rank, base=10000.0, kv_from=None, scale=None):
+    mixer = {"dim": dim, "heads": heads, "kv_rank": kv_rank, "q_rank": q_rank, "rot": {"base": float(base), "dims": rot_dim},
+             "rot_dim": rot_dim, "scale": float(scale if scale is not None else (dim + rot_dim) ** -0.5), "vdim": vdim}
+    if kv_from is not None:
+        mixer["kv_from"] = int(kv_from)
+    return mixer
+
+
+def sogalix_delta(heads, dim):
+    return {"dim": dim, "heads": heads}
+
+
+def sogalix_layer(kind, mixer, ff=None):
+    return {"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": int(ff)} if ff else None}
+
+
+def sogalix_config(width, vocab, layers, eps=1e-6):
+    return {"architecture": "Sogalix", "layers": list(layers), "norm": {"eps": float(eps)}, "vocab": int(vocab), "width": int(width)}
+
+
+def build_sogalix(config, seed=0, gain=1.0, decay_rank=8):
+    """Random tensors {checkpoint name: uint16 bf16 bits} of a Sogalix configuration. decay_rank: inner size of the
+    generalized delta rule's two-step decay projection (the configuration does not name it; the tensors' shapes do)."""
+    rng = np.random.default_rng(seed)
+    W, V = config["width"], config["vocab"]
+    t = {}
+
+    def mat(name, rows, cols, std=None):
+        t[name] = to_bf16(rng.standard_normal((rows, cols)).astype(np.float32) * (std or gain / np.sqrt(cols)))
+
+    def vec(name, n, centre, spread):
+        t[name] = to_bf16((centre + spread * rng.standard_normal(n)).astype(np.float32))
+
+    def norm(name):
+        vec(name, W, 1.0, 0.1)
+        vec(name + ".b", W, 0.0, 0.05)
+
+    mat("embed", V, W, 1.0)
+    norm("embed.norm")
+    norm("final.norm")
+    mat("head", V, W, 4.0 / np.sqrt(W))
+    for i, L in enumerate(config["layers"]):
+        mx, ml, p = L["mixer"], L.get("mlp"), f"l{i}."
+        H, d = mx["heads"], mx["dim"]
+        norm(p + "norm1")
+        if L["type"] == "attention":
+            G, dv = mx["kv_heads"], mx["vdim"]
+            mat(p + "mix.q", H * d, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.k", G * d, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.v", G * dv, W)
+            mat(p + "mix.o", W, H * dv)
+        elif L["type"] == "latent_attention":
+            rd, dv, rq, rk = mx["rot_dim"], mx["vdim"], mx["q_rank"], mx["kv_rank"]
+            mat(p + "mix.dq", rq, W)
+            vec(p + "mix.dq.norm", rq, 1.0, 0.1)
+            mat(p + "mix.uq", H * (d + rd), rq, 2.0 / np.sqrt(rq))
+            if mx.get("kv_from") is None:
+                mat(p + "mix.dkv", rk + rd, W)
+                vec(p + "mix.dkv.norm", rk, 1.0, 0.1)
+            mat(p + "mix.uk", H * d, rk, 2.0 / np.sqrt(rk))
+            mat(p + "mix.uv", H * dv, rk)
+            mat(p + "mix.g", H, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.o", W, H * dv)
+        else:
+            for n in "rkvga":
+                mat(p + "mix." + n, H * d, W)
+            vec(p + "mix.a.b", H * d, 0.0, 0.5)
+            mat(p + "mix.w1", decay_rank, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.w2", H * d, decay_rank, 1.0)
+            vec(p + "mix.w0", H * d, -1.0, 1.0)
+            vec(p + "mix.norm", H * d, 1.0, 0.1)
+            mat(p + "mix.o", W, H * d)
+        if ml is not None:
+            norm(p + "norm2")
+            mat(p + "mlp.up", ml["ff"], W, 2.0 / np.sqrt(W))
+            mat(p + "mlp.down", W, ml["ff"])
+            t[p + "mlp.act"] = to_bf16(np.array([rng.uniform(-1.0, 1.0), rng.uniform(-1.0, 1.0)], np.float32))
+    return t
+
+
 def write_stack_dir(path, config, tensors):
     """config.json + model.safetensors (8-byte little-endian header length, JSON header, data) under `path`."""
     import json
