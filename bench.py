@@ -52,8 +52,9 @@ def parse():
     ap.add_argument("--prompt-len", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=8, help="layers in the CPU-baseline sample")
-    ap.add_argument("--family", default=None, choices=[None, "ralasun", "madalorn"],
-                    help="madalorn: prefill / decode throughput of that layer-list design at --sizes beside a Ralasun model of "
+    ap.add_argument("--family", default=None, choices=[None, "ralasun", "madalorn", "sogalix"],
+                    help="sogalix: prefill / decode throughput of that layer-list design at --sizes beside a Madalorn model of "
+                         "equal size; madalorn: prefill / decode throughput of that layer-list design at --sizes beside a Ralasun model of "
                          "equal size (the closest existing model: same engine, bf16 weights, window attention, routed experts); "
                          "ralasun: prefill / decode throughput of the layer-list family at --sizes beside a Llama model of "
                          "equal size (one GPU; prints its own JSON line; the default workload and line are untouched)")
@@ -230,6 +231,65 @@ def _build_madalorn(S, engine, z, max_pos, rng, pool):
     return m, per_tok / z["layers"]
 
 
+def _build_sogalix(S, engine, z, max_pos, rng, pool):
+    """Latent attention, generalized delta rule, sink attention, generalized delta rule in turn; every second latent layer
+    reads the cache of the latent layer four layers before it. Every layer has the plain feed-forward with as many columns
+    as one token activates in the routed feed-forward of the size. Latent sizes: kv_rank = 4 dim, rot_dim = dim / 2,
+    q_rank = width / 2."""
+    W, V, H, G, d, n = z["width"], z["vocab"], z["heads"], z["kv_heads"], z["dim"], z["layers"]
+    F = z["top"] * z["ff"] + z["shared_ff"]
+    rq, rk, rd, rank = W // 2, 4 * d, d // 2, d
+    layers = []
+    for i in range(n):
+        if i % 4 == 0:
+            mx = S.sogalix_latent(H, d, rd, d, rq, rk, base=250000.0, kv_from=i - 4 if i % 8 == 4 else None)
+            layers.append(S.sogalix_layer("latent_attention", mx, F))
+        elif i % 4 == 2:
+            layers.append(S.sogalix_layer("attention", S.sogalix_attention(H, G, d, d, q_temp=(0.1, 512)), F))
+        else:
+            layers.append(S.sogalix_layer("general_delta", S.sogalix_delta(H, d), F))
+    cfg = S.sogalix_config(W, V, layers)
+    shapes = {f"l{i}.mix.w1": np.empty((rank, 0)) for i in range(n)}
+    m = engine.StackModel(cfg, max_pos, shapes)
+
+    def mat(nm, r, c, std=None):
+        m.set_tensor(nm, _pool_bf16(S, r * c, std or 1.0 / np.sqrt(c), rng, pool).reshape(r, c))
+
+    def vec(nm, k, centre, spread=0.05):
+        m.set_tensor(nm, S.to_bf16((centre + spread * rng.standard_normal(k)).astype(np.float32)))
+
+    def norm(nm):
+        vec(nm, W, 1.0), vec(nm + ".b", W, 0.0)
+
+    mat("embed", V, W, 1.0), mat("head", V, W), norm("embed.norm"), norm("final.norm")
+    per_tok = 0
+    for i, L in enumerate(layers):
+        p, mx = f"l{i}.", L["mixer"]
+        norm(p + "norm1"), norm(p + "norm2")
+        if L["type"] == "latent_attention":
+            own = mx.get("kv_from") is None
+            mat(p + "mix.dq", rq, W), vec(p + "mix.dq.norm", rq, 1.0), mat(p + "mix.uq", H * (d + rd), rq)
+            if own:
+                mat(p + "mix.dkv", rk + rd, W), vec(p + "mix.dkv.norm", rk, 1.0)
+            mat(p + "mix.uk", H * d, rk), mat(p + "mix.uv", H * d, rk), mat(p + "mix.g", H, W), mat(p + "mix.o", W, H * d)
+            # (a chunk that starts the sequence expands as many rows as it has tokens: W_uk and W_uv count once)
+            per_tok += W * (rq + (rk + rd if own else 0) + H) + rq * H * (d + rd) + 2 * rk * H * d + H * d * W
+        elif L["type"] == "attention":
+            mat(p + "mix.q", H * d, W), mat(p + "mix.k", G * d, W), mat(p + "mix.v", G * d, W), mat(p + "mix.o", W, H * d)
+            per_tok += (2 * H * d + 2 * G * d) * W
+        else:
+            for nm in "rkvga":
+                mat(p + "mix." + nm, H * d, W)
+            mat(p + "mix.w1", rank, W), mat(p + "mix.w2", H * d, rank), mat(p + "mix.o", W, H * d)
+            vec(p + "mix.a.b", H * d, 0.0, 0.3), vec(p + "mix.w0", H * d, -1.0, 0.5), vec(p + "mix.norm", H * d, 1.0)
+            per_tok += (6 * H * d + rank) * W + H * d * rank
+        mat(p + "mlp.up", F, W), mat(p + "mlp.down", W, F)
+        m.set_tensor(p + "mlp.act", S.to_bf16(np.array([0.3, -0.2], np.float32)))
+        per_tok += 2 * W * F
+    m.finalize()
+    return m, per_tok / n
+
+
 def stack_bench(args):
     from _pkg import load_package
     pkg = load_package()
@@ -244,6 +304,23 @@ def stack_bench(args):
         z = STACK_SIZES[name]
         W, V = z["width"], z["vocab"]
         max_pos = T + args.steps + args.warmup + 64
+        if args.family == "sogalix":
+            z = dict(z, vdim=z["dim"])
+            t0 = time.time()
+            m, per_tok = _build_sogalix(S, engine, z, max_pos, rng, pool)
+            r = {"size": name, "shape": z, "layers": "latent_attention / general_delta / attention / general_delta in turn",
+                 "load_s": round(time.time() - t0, 1)}
+            got, toks, first = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+            r.update(got)
+            m.free()
+            if not args.no_twin:
+                m, per_tok = _build_madalorn(S, engine, z, max_pos, rng, pool)
+                tw, _, _ = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+                m.free()
+                r["madalorn_twin"] = tw
+            results.append(r)
+            print(json.dumps(r), file=sys.stderr, flush=True)
+            continue
         if args.family == "madalorn":
             # the delta rule's value size equals its key size here, and the attention's values are its keys
             z = dict(z, vdim=z["dim"])
@@ -302,7 +379,9 @@ def stack_bench(args):
             r["llama_twin"] = tw
         results.append(r)
         print(json.dumps(r), file=sys.stderr, flush=True)
-    label = ("layer-list family (Madalorn): prefill / decode tokens/s beside a Ralasun model of equal size"
+    label = ("layer-list family (Sogalix): prefill / decode tokens/s beside a Madalorn model of equal size"
+             if args.family == "sogalix" else
+             "layer-list family (Madalorn): prefill / decode tokens/s beside a Ralasun model of equal size"
              if args.family == "madalorn" else
              "layer-list family (Ralasun): prefill / decode tokens/s beside a Llama model of equal size")
     print(json.dumps({"metric": label, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "prefill_tokens": T,

@@ -239,7 +239,7 @@ int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s) {
   TL_REQUIRE(!a.x_rows || a.x_div >= 1, "dense gemm: x_div must be >= 1");
   TL_REQUIRE(!a.glu || (a.rows & 1) == 0, "dense gemm: gated pairs need an even number of rows (got %d)", a.rows);
   const int groups = a.groups > 0 ? a.groups : 1;
-  TL_REQUIRE(groups == 1 || a.group_off || (a.x_gstride > 0 && a.y_gstride > 0 && !a.x_rows && !a.y_rows),
+  TL_REQUIRE(groups == 1 || a.group_off || (a.x_gstride >= 0 && a.y_gstride > 0 && !a.x_rows && !a.y_rows),
              "dense gemm: groups without group_off or per-head column strides");
   TL_REQUIRE(!a.act || !a.glu, "dense gemm: an activation and a gated unit in one epilogue");
   // 128 x 128 tiles when there is enough of both sides to fill them (grouped launches: tokens per group on average)

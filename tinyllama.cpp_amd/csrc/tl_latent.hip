@@ -5,9 +5,14 @@
 //   score            q_plain,n . (W_uk,n c) + q_rot,n . k_rot  =  (W_uk,n^T q_plain,n) . c + q_rot,n . k_rot
 //   output           sum_j p_j W_uv,n c_j  =  W_uv,n (sum_j p_j c_j)
 //
-// so attention runs over the CACHE ROWS themselves (tl_swa.hip with one key/value "head": key = the whole row, value = its
+// so for one token, or a few, attention runs over the CACHE ROWS themselves (tl_swa.hip with one key/value "head": key = the whole row, value = its
 // first kv_rank columns), with the query of head n absorbed through W_uk,n^T in front and W_uv,n applied to the weighted sum
-// of latents behind (both are one product per head, tl_dense.hip). Nothing per head is ever expanded over the context.
+// of latents behind (both are one product per head, tl_dense.hip): nothing per head is expanded over the context, and a
+// decode step reads kv_rank + rot_dim floats per cached token instead of heads * (dim + rot_dim + vdim).
+// A long prompt chunk is the other way round: its cost is the products per (query, key) pair, which the absorbed form makes
+// (kv_rank + rot_dim + kv_rank) / (dim + rot_dim + vdim) times as many. There the engine expands keys and values per head for
+// the rows the chunk can see (two matrix-core products over the cache rows, latent_spread for the shared rotated part) and
+// runs ordinary attention with as many key heads as query heads.
 //
 //   latent_post    per token: the query latent is RMS-normed in place (plain weights); the key/value latent is RMS-normed and,
 //                  with the rotated shared key part behind it, written to row `pos` of the cache.
@@ -78,8 +83,8 @@ __global__ __launch_bounds__(256) void latent_query_kernel(const LatentQueryArgs
   const int t = blockIdx.x, n = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (n >= a.heads) return;
   const int pos = (a.pos_dev ? *a.pos_dev : a.start_pos) + t;
-  const float* src = a.q + ((size_t)t * a.heads + n) * (a.dim + a.rot_dim) + a.dim;
-  float* dst = a.qa + ((size_t)t * a.heads + n) * (a.kv_rank + a.rot_dim) + a.kv_rank;
+  const float* src = a.q + ((size_t)t * a.heads + n) * a.q_stride + a.q_off;
+  float* dst = a.out + ((size_t)t * a.heads + n) * a.out_stride + a.out_off;
   for (int i = lane; 2 * i < a.rot_dim; i += 64) {
     const int d0 = 2 * i, d1 = d0 + 1;
     float u = src[d0], v = d1 < a.rot_dim ? src[d1] : 0.0f;
@@ -93,6 +98,16 @@ __global__ __launch_bounds__(256) void latent_query_kernel(const LatentQueryArgs
     dst[d0] = u;
     if (d1 < a.rot_dim) dst[d1] = v;
   }
+}
+
+__global__ __launch_bounds__(256) void latent_spread_kernel(const float* __restrict__ cache, int kv_rank, int rot_dim,
+                                                           float* __restrict__ k, int heads, int dim, long long total) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // (row, head, rotated dimension)
+  if (i >= total) return;
+  const int r = (int)(i % rot_dim);
+  const long long ph = i / rot_dim;
+  const long long p = ph / heads;
+  k[ph * (dim + rot_dim) + dim + r] = cache[p * (kv_rank + rot_dim) + kv_rank + r];
 }
 
 __global__ __launch_bounds__(256) void head_gate_kernel(float* __restrict__ o, const float* __restrict__ gate, int gate_ld,
@@ -119,13 +134,24 @@ int tl_launch_latent_post(const LatentPostArgs& a, hipStream_t s) {
 }
 
 int tl_launch_latent_query(const LatentQueryArgs& a, hipStream_t s) {
-  TL_REQUIRE(a.q && a.qa && a.T > 0 && a.heads > 0 && a.dim > 0 && a.kv_rank > 0 && a.rot_dim >= 0, "latent_query: bad arguments");
+  TL_REQUIRE(a.q && a.out && a.T > 0 && a.heads > 0 && a.rot_dim >= 0 && a.q_off >= 0 && a.out_off >= 0 &&
+                 a.q_stride >= a.q_off + a.rot_dim && a.out_stride >= a.out_off + a.rot_dim,
+             "latent_query: bad arguments");
   TL_REQUIRE(a.rot_dims >= 0 && a.rot_dims <= a.rot_dim && (a.rot_dims & 1) == 0 && (a.rot_dims == 0 || a.freq),
              "latent_query: %d turning dimensions of %d", a.rot_dims, a.rot_dim);
   if (a.rot_dim == 0) return 0;
   const int per_token = (a.heads + 3) / 4;
   TL_REQUIRE(per_token <= 65535, "latent_query: too many heads");
   latent_query_kernel<<<dim3(a.T, per_token), 256, 0, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_latent_spread(const float* cache, int kv_rank, int rot_dim, float* k, int heads, int dim, int P, hipStream_t s) {
+  TL_REQUIRE(cache && k && kv_rank > 0 && rot_dim >= 0 && heads > 0 && dim > 0 && P > 0, "latent_spread: bad arguments");
+  if (rot_dim == 0) return 0;
+  const long long total = (long long)P * heads * rot_dim;
+  latent_spread_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(cache, kv_rank, rot_dim, k, heads, dim, total);
   TL_HIP(hipGetLastError());
   return 0;
 }

@@ -41,7 +41,7 @@ struct DenseArgs {
   int act, act_from;
   float act_p, act_q;
   // groups > 1 without group_off: one product per head over ALL items -- group g multiplies matrix g with the columns
-  // x[.][g * x_gstride ..] and writes y[.][g * y_gstride ..]
+  // x[.][g * x_gstride ..] (0: every head reads the same columns) and writes y[.][g * y_gstride ..]
   int x_gstride, y_gstride;
 };
 int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s);
@@ -205,14 +205,19 @@ struct LatentPostArgs {
 };
 int tl_launch_latent_post(const LatentPostArgs& a, hipStream_t s);
 struct LatentQueryArgs {
-  const float* q;        // [T][heads * (dim + rot_dim)]: per head dim plain | rot_dim to be rotated
-  float* qa;             // [T][heads * (kv_rank + rot_dim)]: the rotated part goes behind each head's kv_rank absorbed columns
-  int heads, dim, rot_dim, kv_rank, rot_dims;
+  const float* q;        // [T][heads * q_stride]: head n's part to be rotated starts at column n * q_stride + q_off
+  int q_stride, q_off;
+  float* out;            // [T][heads * out_stride]: it goes to column n * out_stride + out_off (may be q itself: in place)
+  int out_stride, out_off;
+  int heads, rot_dim, rot_dims;
   const double* freq;
   int T, start_pos;
   const int* pos_dev;
 };
 int tl_launch_latent_query(const LatentQueryArgs& a, hipStream_t s);
+// keys per head for a prompt chunk: k[p][n * (dim + rot_dim) + dim ..] = the rotated part of cache row p, for every head n and
+// the rows p < P (the plain parts in front come from a product per head over the same rows)
+int tl_launch_latent_spread(const float* cache, int kv_rank, int rot_dim, float* k, int heads, int dim, int P, hipStream_t s);
 // o[t][n][:] *= sigmoid(gate[t * gate_ld + n]) for the heads n of a token; o [T][heads * vdim]
 int tl_launch_head_gate(float* o, const float* gate, int gate_ld, int T, int heads, int vdim, hipStream_t s);
 

@@ -67,8 +67,9 @@ struct Layer {
   float *state = nullptr, *hist = nullptr;   // delta rule: S and the convolution's history
   float *norm2_b = nullptr;                  // layer norm
   // latent attention: wqkv = dq | dkv | g stacked; wuq [heads * (dim + rot_dim)][q_rank]; wukt [heads][kv_rank][dim] (the
-  // TRANSPOSE of each head's block of mix.uk: the query is absorbed through it); wuv [heads][vdim][kv_rank] as stored
-  uint16_t *wuq = nullptr, *wukt = nullptr, *wuv = nullptr;
+  // TRANSPOSE of each head's block of mix.uk: the query of a decode step is absorbed through it); wuv [heads][vdim][kv_rank]
+  // as stored
+  uint16_t *wuq = nullptr, *wuk = nullptr, *wukt = nullptr, *wuv = nullptr;  // (wuk as stored: the expanded keys of a chunk)
   float *dq_norm = nullptr, *dkv_norm = nullptr;
   float* ckv = nullptr;                      // cache rows [max_pos][kv_rank + rot_dim] (an owner's; kv_src's otherwise)
   int kv_src = -1;                           // the latent layer whose cache this one reads (itself unless kv_from)
@@ -107,6 +108,9 @@ struct TlStack {
   float* h = nullptr;       // norm-first blocks: the normalised input both sublayers read
   float *dq = nullptr, *da = nullptr, *dg = nullptr, *dbeta = nullptr, *ddecay = nullptr;  // delta rule
   float *lq = nullptr, *lqa = nullptr;      // latent attention: up-projected queries, absorbed queries
+  float *lk = nullptr, *lv = nullptr;       // ... and, for long chunks, keys / values per head of every row the chunk sees
+  int max_lk = 0, max_lv = 0;
+  int latent_expand = 64;                   // chunks of at least this many tokens expand (TL_STACK_LATENT_EXPAND; 0: never)
   float *gw = nullptr, *gu = nullptr, *gau = nullptr, *grau = nullptr, *grk = nullptr;  // generalized delta rule (gdelta_pre)
   int max_lq = 0, max_lqa = 0, max_gd = 0, gdelta_layers = 0;
   float *act_buf = nullptr, *eout = nullptr, *sact = nullptr, *sout = nullptr, *sgate = nullptr;
@@ -312,12 +316,15 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
       if (own_kv) st->cache_bytes += sizeof(float) * (size_t)cfg->max_positions * L.kd;
       st->max_lq = L.qd > st->max_lq ? L.qd : st->max_lq;
       st->max_lqa = sp.heads * ah > st->max_lqa ? sp.heads * ah : st->max_lqa;
+      st->max_lk = sp.heads * qh > st->max_lk ? sp.heads * qh : st->max_lk;
+      st->max_lv = sp.heads * sp.vdim > st->max_lv ? sp.heads * sp.vdim : st->max_lv;
       st->max_od = sp.heads * sp.kv_rank > st->max_od ? sp.heads * sp.kv_rank : st->max_od;  // the weighted latents of all heads
       L.expect.insert({"mix.dq", "mix.dq.norm", "mix.uq", "mix.uk", "mix.uv", "mix.o"});
       if (own_kv) L.expect.insert({"mix.dkv", "mix.dkv.norm"});
       if (sp.head_gate) L.expect.insert("mix.g");
       if ((rc = dev_alloc(st, &L.wuq, (size_t)L.qd * sp.q_rank))) break;
       if ((rc = dev_alloc(st, &L.wukt, (size_t)sp.heads * sp.kv_rank * sp.dim))) break;
+      if ((rc = dev_alloc(st, &L.wuk, (size_t)sp.heads * sp.kv_rank * sp.dim))) break;
       if ((rc = dev_alloc(st, &L.wuv, (size_t)sp.heads * sp.vdim * sp.kv_rank))) break;
       if ((rc = dev_alloc(st, &L.dq_norm, sp.q_rank))) break;
       if ((rc = dev_alloc(st, &L.dkv_norm, sp.kv_rank))) break;
@@ -464,6 +471,7 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
   if (const char* e = getenv("TL_STACK_GEMV")) st->gemv_decode = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FUSE_ROUTER")) st->fuse_router = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FORK")) st->fork = atoi(e) != 0;
+  if (const char* e = getenv("TL_STACK_LATENT_EXPAND")) st->latent_expand = atoi(e) > 0 ? atoi(e) : 0;
   *out = st;
   return 0;
 }
@@ -547,6 +555,7 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
         for (int d = 0; d < sp.dim; ++d)
           for (int c = 0; c < sp.kv_rank; ++c)
             tr[((size_t)hh * sp.kv_rank + c) * sp.dim + d] = src[((size_t)hh * sp.dim + d) * sp.kv_rank + c];
+      TL_TRY(upload_bf16(L.wuk, host, tr.size(), s));
       return upload_bf16(L.wukt, tr.data(), tr.size(), s);
     }
   }
@@ -694,6 +703,10 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
   if (st->max_lq) {
     TL_TRY(dev_alloc(st, &st->lq, C * st->max_lq));
     TL_TRY(dev_alloc(st, &st->lqa, C * st->max_lqa));
+    if (st->latent_expand > 0) {
+      TL_TRY(dev_alloc(st, &st->lk, (size_t)st->cfg.max_positions * st->max_lk));
+      TL_TRY(dev_alloc(st, &st->lv, (size_t)st->cfg.max_positions * st->max_lv));
+    }
   }
   if (st->max_gd) {
     TL_TRY(dev_alloc(st, &st->da, C * st->max_gd));
@@ -1158,20 +1171,51 @@ int latent_mixer(TlStack* st, Layer& L, const float* in, int T, int start_pos, c
   p.pos_dev = pos_dev;
   TL_TRY(tl_launch_latent_post(p, s));
   TL_TRY(project(st, L.wuq, L.qd, sp.q_rank, st->qkv, ld, st->lq, L.qd, T, s));
-  // the plain part of head n's query through W_uk,n^T: scores against the cached latent itself
-  TL_TRY(project_heads(st, L.wukt, H, sp.kv_rank, sp.dim, st->lq, L.qd, qh, st->lqa, H * ah, ah, T, s));
   LatentQueryArgs q = {};
   q.q = st->lq;
-  q.qa = st->lqa;
+  q.q_stride = qh;
+  q.q_off = sp.dim;
   q.heads = H;
-  q.dim = sp.dim;
   q.rot_dim = sp.rot_dim;
-  q.kv_rank = sp.kv_rank;
   q.rot_dims = sp.rot_dims;
   q.freq = L.freq;
   q.T = T;
   q.start_pos = start_pos;
   q.pos_dev = pos_dev;
+  if (!pos_dev && st->latent_expand > 0 && T >= st->latent_expand) {
+    // A long chunk: keys [W_uk,n c | rotated part] and values W_uv,n c per head for the rows [0, start_pos + T), then ordinary
+    // attention with as many key heads as query heads (fewer products per query-key pair than over the latent rows).
+    const int P = start_pos + T;
+    q.out = st->lq;  // the rotated query part in place
+    q.out_stride = qh;
+    q.out_off = sp.dim;
+    TL_TRY(tl_launch_latent_query(q, s));
+    TL_TRY(project_heads(st, L.wuk, H, sp.dim, sp.kv_rank, L.ckv, ah, 0, st->lk, H * qh, qh, P, s));
+    TL_TRY(tl_launch_latent_spread(L.ckv, sp.kv_rank, sp.rot_dim, st->lk, H, sp.dim, P, s));
+    TL_TRY(project(st, L.wuv, H * sp.vdim, sp.kv_rank, L.ckv, ah, st->lv, H * sp.vdim, P, s));
+    SwaArgs e = {};
+    e.q = st->lq;
+    e.ldq = H * qh;
+    e.kc = st->lk;
+    e.vc = st->lv;
+    e.out = st->att;
+    e.T = T;
+    e.heads = H;
+    e.kv_heads = H;
+    e.dim = qh;
+    e.vdim = sp.vdim;
+    e.scale = sp.scale;
+    e.start_pos = start_pos;
+    e.nsplit = 1;
+    TL_TRY(tl_launch_swa(e, s));
+    if (sp.head_gate) TL_TRY(tl_launch_head_gate(st->att, st->qkv + L.gate_off, ld, T, H, sp.vdim, s));
+    return project(st, L.wo, W, L.od, st->att, L.od, st->proj, W, T, s);
+  }
+  // the plain part of head n's query through W_uk,n^T: scores against the cached latent itself
+  TL_TRY(project_heads(st, L.wukt, H, sp.kv_rank, sp.dim, st->lq, L.qd, qh, st->lqa, H * ah, ah, T, s));
+  q.out = st->lqa;  // the rotated part behind each head's absorbed columns
+  q.out_stride = ah;
+  q.out_off = sp.kv_rank;
   TL_TRY(tl_launch_latent_query(q, s));
   SwaArgs a = {};
   a.q = st->lqa;
