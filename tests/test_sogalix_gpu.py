@@ -412,6 +412,28 @@ def test_far_keys_decide_the_logits(env):
     m.free()
 
 
+def test_two_forms_of_latent_attention_agree(env):
+    """Attention over the cached latent rows themselves (queries absorbed through W_uk^T, W_uv behind the weighted sum) and
+    ordinary attention over keys and values expanded per head are the same sum: a model that never expands, one that
+    expands from 16 tokens on, and the oracle, on a prompt cut so that later portions see rows earlier portions wrote."""
+    cfg = small_config(env["synth"], "wide")
+    tensors = env["synth"].build_sogalix(cfg, 47)
+    absorbed, _, orc = make(env, cfg, tensors=tensors, TL_STACK_LATENT_EXPAND=0)
+    expanded, _, _ = make(env, cfg, tensors=tensors, TL_STACK_LATENT_EXPAND=16)
+    toks = np.random.default_rng(9).integers(0, cfg["vocab"], 260).astype(np.int32)
+    want = orc.forward(list(toks))
+    outs = []
+    for m in (absorbed, expanded):
+        got, p = [], 0
+        for n in (70, 16, 5, 100, 33, 36):
+            got.append(m.prefill_rows(toks[p:p + n], p))
+            p += n
+        outs.append(np.concatenate(got))
+        assert rel_rms(outs[-1], want) < FP32_TOL
+        m.free()
+    assert rel_rms(outs[0], outs[1]) < FP32_TOL and not np.array_equal(outs[0], outs[1])   # (two code paths, not one)
+
+
 def test_long_decoding_and_device_loops(env):
     """Greedy generation on the device (graph replays back to back) equals the oracle's token-by-token arg-max; the sampled
     loop is reproducible by seed and stays inside the vocabulary."""
