@@ -515,6 +515,43 @@ def test_generation_through_the_host_session(env, tmp_path):
         hostapi.Session(str(tmp_path / "bad"), 0, 64)
 
 
+def test_schedule_replayed_by_the_trace_program(env, tmp_path):
+    """The command-line program that replays a recorded schedule (JSON lines on standard input: per step the next tokens of a
+    request and the places whose logits are wanted) over a checkpoint folder: a whole prompt, then a second request in
+    portions and single tokens after the first one gave its cache back; both number formats against the oracle."""
+    import subprocess
+    synth = env["synth"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tinyllama.cpp_amd", "host", "tl_trace")
+    assert os.path.exists(exe), "build the host layer first (make -C tinyllama.cpp_amd/host)"
+    cfg = small_config(synth, "mixed")
+    tensors = synth.build_sogalix(cfg, 53, decay_rank=4)
+    synth.write_stack_dir(str(tmp_path / "ckpt"), cfg, tensors)
+    orc = env["oracle"].SogalixOracle(cfg, tensors)
+    rng = np.random.default_rng(11)
+    a = [int(t) for t in rng.integers(0, cfg["vocab"], 90)]
+    b = [int(t) for t in rng.integers(0, cfg["vocab"], 70)]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a, "want": [0, 1, 40, 89]}], "end": ["a"]},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:37], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[37:39], "want": [0, 1]}], "end": []}]
+    steps += [{"step": 3 + i, "entries": [{"id": "b", "tokens": [b[39 + i]], "want": [0]}], "end": ["b"] if 39 + i == 69 else []}
+              for i in range(31)]
+    want_a = orc.forward(a)[[0, 1, 40, 89]]
+    orc.reset()
+    want_b = orc.forward(b)[37:]
+    for dtype, tol in (("float32", FP32_TOL), ("bfloat16", BF16_TOL)):
+        out = tmp_path / dtype
+        out.mkdir()
+        r = subprocess.run([exe, "--model", str(tmp_path / "ckpt"), "--dtype", dtype, "--out", str(out), "--max-tokens", "96"],
+                           input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=100)
+        assert r.returncode == 0, r.stderr
+        assert [ln for ln in r.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(len(steps))]
+        assert not (out / "1.f32").exists()                       # nothing was wanted in that step
+        got_a = np.fromfile(out / "0.f32", np.float32).reshape(4, cfg["vocab"])
+        got_b = np.concatenate([np.fromfile(out / f"{i}.f32", np.float32).reshape(-1, cfg["vocab"]) for i in range(2, len(steps))])
+        assert rel_rms(got_a, want_a) < tol and rel_rms(got_b, want_b) < tol, dtype
+
+
 def random_config(synth, seed):
     """A configuration drawn at random: layer order, head counts and group ratios, head sizes (also indivisible by 4 and above
     128), latent sizes, rotated sizes, temperature steps, shared caches, with and without feed-forward."""

@@ -497,7 +497,8 @@ def _sogalix_spec(sp, i, L, tensors):
     mx, ml = L["mixer"], L.get("mlp")
     sp.block, sp.heads, sp.dim = 2, mx["heads"], mx["dim"]
     if L["type"] == "attention":
-        sp.mixer, sp.kv_heads, sp.vdim, sp.scale, sp.attn_weight = 0, mx["kv_heads"], mx["vdim"], float(mx["scale"]), 2
+        sp.mixer, sp.kv_heads, sp.vdim = 0, mx.get("kv_heads", mx["heads"]), mx.get("vdim", mx["dim"])
+        sp.scale, sp.attn_weight = float(mx["scale"]), 2
         qt = mx.get("q_temp")
         if qt:
             sp.q_temp_coef, sp.q_temp_every = float(qt["coef"]), int(qt["every"])

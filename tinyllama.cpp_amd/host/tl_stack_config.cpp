@@ -195,8 +195,8 @@ tl_layer_spec sogalix_layer(const Json& layers, int index, const SafeTensorsFile
   sp.dim = geti(mx, "dim");
   if (type == "attention") {
     sp.mixer = TL_MIXER_SWA;
-    sp.kv_heads = geti(mx, "kv_heads");
-    sp.vdim = geti(mx, "vdim");
+    sp.kv_heads = present(mx, "kv_heads") ? geti(mx, "kv_heads") : sp.heads;  // (no entry: a key/value head per query head)
+    sp.vdim = present(mx, "vdim") ? geti(mx, "vdim") : sp.dim;
     sp.scale = getf(mx, "scale");
     sp.attn_weight = TL_ATTN_SOFTMAX_SINK;  // the sink is part of the design
     if (const Json* qt = present(mx, "q_temp")) {
