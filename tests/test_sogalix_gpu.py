@@ -434,6 +434,28 @@ def test_two_forms_of_latent_attention_agree(env):
     assert rel_rms(outs[0], outs[1]) < FP32_TOL and not np.array_equal(outs[0], outs[1])   # (two code paths, not one)
 
 
+def test_short_portions_and_first_tokens_multiply_exactly(env):
+    """With bf16 activations in the chunk products, a portion of fewer than 64 tokens still multiplies FP32-grade, and a long
+    prompt's first token goes through on its own on the one-token path (the first token's read-out of the generalized delta
+    rule is a unit vector whose sign can hang on the last bits of its input): that row matches the oracle at FP32 accuracy,
+    the rest at bf16's. TL_STACK_LEAD=0 switches the second part off."""
+    cfg = small_config(env["synth"], "mixed")
+    tensors = env["synth"].build_sogalix(cfg, 59)
+    toks = np.random.default_rng(10).integers(0, cfg["vocab"], 140).astype(np.int32)
+    m, _, orc = make(env, cfg, tensors=tensors, exact=False)
+    want = orc.forward(list(toks))
+    got = m.prefill_rows(toks, 0)
+    assert rel_rms(got[:1], want[:1]) < FP32_TOL and FP32_TOL < rel_rms(got[1:], want[1:]) < BF16_TOL
+    m.reset_kv()
+    short = np.concatenate([m.prefill_rows(toks[:40], 0), m.prefill_rows(toks[40:63], 40)])
+    assert rel_rms(short, want[:63]) < FP32_TOL
+    m.free()
+    m, _, _ = make(env, cfg, tensors=tensors, exact=False, TL_STACK_LEAD=0)
+    got = m.prefill_rows(toks, 0)
+    assert FP32_TOL < rel_rms(got[:1], want[:1]) < BF16_TOL
+    m.free()
+
+
 def test_long_decoding_and_device_loops(env):
     """Greedy generation on the device (graph replays back to back) equals the oracle's token-by-token arg-max; the sampled
     loop is reproducible by seed and stays inside the vocabulary."""

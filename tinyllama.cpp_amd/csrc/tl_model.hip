@@ -1989,8 +1989,11 @@ extern "C" int tl_model_prefill_rows(tl_model* m, const int* tokens_host, int nu
     m->pf.rows_cap = need;
   }
   int r0 = 0;
-  for (int t0 = 0; t0 < num_tokens; t0 += C) {
-    const int T = num_tokens - t0 < C ? num_tokens - t0 : C;
+  // (a design may ask for the first tokens of a sequence as a short portion of their own: tl_stack_lead_tokens)
+  const int lead = tl_stack_lead_tokens(m->stack, num_tokens, start_pos);
+  for (int t0 = 0, T = 0; t0 < num_tokens; t0 += T) {
+    T = num_tokens - t0 < C ? num_tokens - t0 : C;
+    if (t0 == 0 && lead > 0) T = lead;
     int r1 = r0;
     while (r1 < n_rows && rows[r1] < t0 + T) ++r1;
     std::vector<int> local(rows.begin() + r0, rows.begin() + r1);

@@ -355,6 +355,9 @@ int tl_stack_set_terms(TlStack* st, int terms);
 int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, const int* pos_dev, const int* rows_dev,
                      int n_rows, float* logits_dev, hipStream_t s);
 int tl_stack_chunk(const TlStack* st);
+// > 0: a prompt of num_tokens at start_pos should run its first so many tokens as a portion of their own (short portions
+// multiply FP32-grade whatever the chunks use); 0: no such wish
+int tl_stack_lead_tokens(const TlStack* st, int num_tokens, int start_pos);
 int tl_stack_cache_ptr(TlStack* st, int which, int layer, void** out);
 // residual stream of the last forward call, [T][width] (tests)
 const float* tl_stack_residual(const TlStack* st);

@@ -95,6 +95,8 @@ struct TlStack {
   // at 512, 140.4 k at 1024, 171.6 k at 2048 -- the experts' grouped GEMMs see 4 x the tokens per expert, the dense ones
   // enough tiles for the 128 x 128 shape.
   int chunk = 2048;
+  int lead = 1;             // tokens of tl_stack_lead_tokens (TL_STACK_LEAD; 0: none)
+  int exact_below = 64;     // portions shorter than this always multiply with three terms (TL_STACK_EXACT_BELOW; at least 2)
   bool gemv_decode = true;
   bool fuse_router = true;  // TL_STACK_FUSE_ROUTER=0: the router as a launch of its own (A/B, tests)
   // One token through a parallel block: mixer and feed-forward read the same h and meet only in the residual sum, so the
@@ -471,6 +473,8 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
   if (const char* e = getenv("TL_STACK_GEMV")) st->gemv_decode = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FUSE_ROUTER")) st->fuse_router = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FORK")) st->fork = atoi(e) != 0;
+  if (const char* e = getenv("TL_STACK_LEAD")) st->lead = atoi(e) > 0 ? atoi(e) : 0;
+  if (const char* e = getenv("TL_STACK_EXACT_BELOW")) st->exact_below = atoi(e) > 2 ? atoi(e) : 2;
   if (const char* e = getenv("TL_STACK_LATENT_EXPAND")) st->latent_expand = atoi(e) > 0 ? atoi(e) : 0;
   *out = st;
   return 0;
@@ -776,6 +780,19 @@ int tl_stack_set_terms(TlStack* st, int terms) {
 }
 
 int tl_stack_chunk(const TlStack* st) { return st->chunk; }
+
+// The generalized delta rule starts from S = 0: the first token leaves S = k v^T, its read-out is v (k . r), and the head norm
+// behind it turns that into +-v / rms(v), softened only by eps. Where k . r happens to be small the SIGN hangs on the last
+// bits of the layer's input, bf16 rounding of the activations in front moves the residual stream at position 0 by tens of
+// percent (measured: 24 % of its size, against 0.3 % at later positions), and every early position attends to that token.
+// So a sequence's first token goes through on its own, on the one-token path (FP32 GEMVs): one more pass over the weights per
+// prompt, the cost of a decode step. (Sixteen tokens as a three-term chunk were measured first: such a chunk fills a third of
+// the chip and cost a fifth of the prefill rate; the second token is five times less sensitive than the first, the third not
+// at all.)
+int tl_stack_lead_tokens(const TlStack* st, int num_tokens, int start_pos) {
+  if (start_pos != 0 || st->lead <= 0 || st->gdelta_layers == 0 || st->terms == 3) return 0;
+  return num_tokens >= st->exact_below && num_tokens > st->lead ? st->lead : 0;
+}
 const float* tl_stack_residual(const TlStack* st) { return st->x; }
 void tl_stack_set_layer_hook(TlStack* st, tl_stack_layer_hook hook, void* ctx) {
   st->hook = hook;
@@ -833,7 +850,10 @@ namespace {
 // One token is always FP32-grade: the decode step's GEMVs are, and where TL_STACK_GEMV=0 sends it through the chunk GEMMs
 // instead (a test configuration) it takes three terms, whatever the chunks use; so the captured step never depends on a
 // setting that may change after the capture.
-inline int terms_for(const TlStack* st, int T) { return T == 1 ? 3 : st->terms; }
+// The same holds for every portion of fewer than exact_below tokens (one token tile of the small GEMM shape): such a product
+// is bound by reading its weights, three terms cost it nothing, and a short portion then agrees with the same tokens decoded
+// one by one to FP32 accuracy instead of bf16's.
+inline int terms_for(const TlStack* st, int T) { return T < st->exact_below ? 3 : st->terms; }
 
 // y[T][rows] = x[T][cols] W^T for a chunk, or the GEMV for the one token of a decode step
 int project(TlStack* st, const uint16_t* w, int rows, int cols, const float* x, int ldx, float* y, int ldy, int T,
