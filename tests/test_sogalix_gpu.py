@@ -90,10 +90,6 @@ def sync(env):
     env["capi"].check(env["capi"].lib().tl_device_sync(), "sync")
 
 
-def bf16_round(synth, a):
-    return synth.from_bf16(synth.to_bf16(np.asarray(a, np.float32)))
-
-
 # ---- each mechanism alone ---------------------------------------------------------------------------------------------
 def test_layer_norm(env):
     capi = env["capi"]
