@@ -249,13 +249,16 @@ enum tl_mixer_kind {
   TL_MIXER_LATENT = 2,      /* attention over a cached latent: queries through a normalised latent, keys and values of all heads
                                up-projected from one normalised latent per token, plus one rotated key part shared by the heads;
                                the cache holds the latent and that part only (optionally another layer's, kv_from) */
-  TL_MIXER_GDELTA = 3       /* generalized delta rule: decay and removal rate per key channel,
+  TL_MIXER_GDELTA = 3,      /* generalized delta rule: decay and removal rate per key channel,
                                S <- diag(w) S - (a u)(u^T S) + k v^T with the unit key u, o = S^T r */
+  TL_MIXER_LINEAR = 4       /* gated linear attention whose forget gate also decides what is written (no keys):
+                               q = silu(W_q h), f = l + (1 - l) sigmoid(W_f h + b), S <- diag(f) S + (1 - f) v^T, o = S^T q,
+                               RMS norm per head with one plain weight [vdim] */
 };
 enum tl_mlp_kind {
   TL_MLP_NONE = 0,
   TL_MLP_MOE = 1,           /* routed experts (+ shared expert) */
-  TL_MLP_DENSE = 2,         /* one gated unit */
+  TL_MLP_DENSE = 2,         /* one gated unit (tl_glu_kind) */
   TL_MLP_UNIT = 3           /* W_down act(W_up h): no gate; act = tl_act_kind (shared_ff is its size) */
 };
 enum tl_act_kind {
@@ -263,6 +266,10 @@ enum tl_act_kind {
   TL_ACT_XIELU = 1,         /* z > 0: P z^2 + z / 2; z <= 0: Q (e^z - 1 - z) + z / 2, with P = softplus(p), Q = 1/2 + softplus(q)
                                from the two numbers of the tensor mlp.act */
   TL_ACT_TANH = 2
+};
+enum tl_glu_kind {
+  TL_GLU_SWISH = 0,         /* g sigmoid(act_alpha g) (u + glu_up_add), g = min(gate, limit), u = clamp(up, -limit, limit) */
+  TL_GLU_RELU = 1           /* max(gate, 0) * up */
 };
 enum tl_block_kind {
   TL_BLOCK_POST_NORM = 0,   /* x += N1(mixer(x)); x += N2(ff(x)): the sublayers read x, the norm is on their output */
@@ -272,23 +279,30 @@ enum tl_block_kind {
 enum tl_norm_kind {
   TL_NORM_RMS_ONE_PLUS = 0, /* y / sqrt(mean(y^2) + eps) * (1 + w) */
   TL_NORM_DYT = 1,          /* tanh(alpha y) * w + b: elementwise, no mean or variance (tensors <name>, <name>.alpha, <name>.b) */
-  TL_NORM_LAYER = 2         /* (y - mean) / sqrt(var + eps) * w + b, var = mean of the squared deviations (tensors <name>, <name>.b) */
+  TL_NORM_LAYER = 2,        /* (y - mean) / sqrt(var + eps) * w + b, var = mean of the squared deviations (tensors <name>, <name>.b) */
+  TL_NORM_RMS = 3           /* y / sqrt(mean(y^2) + eps) * w: plain weights (pre-norm blocks) */
 };
 enum tl_attn_weight {
   TL_ATTN_SOFTMAX = 0,      /* weights normalised over the visible keys */
   TL_ATTN_SIGMOID = 1,      /* weight of a visible key = sigmoid(score + bias[head]); not normalised */
-  TL_ATTN_SOFTMAX_SINK = 2  /* softmax with one more term in the denominator: a sink of score 0 that carries no value */
+  TL_ATTN_SOFTMAX_SINK = 2, /* softmax with one more term in the denominator: a sink of score 0 that carries no value */
+  TL_ATTN_SOFTMAX_LEARNED_SINK = 3 /* the same with exp(sink[head]) as that term: a learned number per head (mix.sink) */
 };
 enum tl_qk_norm {
   TL_QK_NORM_NONE = 0,
   TL_QK_NORM_WHOLE = 1,     /* RMS norm over the WHOLE q and the whole k projection, plain weights (mix.q.norm, mix.k.norm) */
-  TL_QK_NORM_HEAD_UNIT = 2  /* per head, after the rotation: x / sqrt(mean(x^2) + eps), no weights */
+  TL_QK_NORM_HEAD_UNIT = 2, /* per head, after the rotation: x / sqrt(mean(x^2) + eps), no weights */
+  TL_QK_NORM_HEAD_RMS = 3   /* per head (and score map): RMS norm over dim with one plain weight [dim] for all heads
+                               (mix.q.norm, mix.k.norm) */
 };
 enum tl_route_kind {
   TL_ROUTE_TOP_LOGITS = 0,  /* the `top` largest logits (+ bias); weights = softmax over the chosen logits */
-  TL_ROUTE_SOFTMAX_GROUPS = 1 /* scores = softmax over all experts; experts in `route_groups` equal groups of neighbours, a
+  TL_ROUTE_SOFTMAX_GROUPS = 1, /* scores = softmax over all experts; experts in `route_groups` equal groups of neighbours, a
                                group's score its best expert's, only the best `route_keep` groups can be chosen from;
                                weights = the chosen scores divided by their sum (+ 1e-20) */
+  TL_ROUTE_SIGMOID_GROUPS = 2 /* scores = sigmoid(logits); choice = score + mlp.correction[expert]; a group's rank is the sum of
+                               its two best choices, experts outside the best `route_keep` groups cannot be chosen; the `top`
+                               best choices are taken; weights = their scores (without the correction, not normalised) */
 };
 typedef struct tl_layer_spec {
   int mixer;                /* tl_mixer_kind */
@@ -336,6 +350,27 @@ typedef struct tl_layer_spec {
   int head_gate;            /* TL_MIXER_LATENT: 1: head n's output is multiplied by sigmoid(W_g h)_n (mix.g, one row per head) */
   float decay_scale;        /* TL_MIXER_GDELTA: decay = exp(-decay_scale * sigmoid(W_w2 tanh(W_w1 h) + w0)); decay_rank = rows of w1 */
   int act;                  /* TL_MLP_UNIT: tl_act_kind */
+  int glu;                  /* tl_glu_kind of the gated units (experts, shared expert, dense unit) */
+  /* ---- TL_MIXER_SWA, all zero = none of it ---- */
+  int score_maps;           /* 2: differential attention -- q and k hold two maps per head ([map 1 | map 2], dim each) over the
+                               same values; o = a1 - lambda a2 with lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff_init (tensors
+                               mix.lq1 .. mix.lk2 [dim]), then o / rms(o) over vdim (no weight) times (1 - diff_init) */
+  float diff_init;
+  int out_gate;             /* 1: the concatenated heads are multiplied by sigmoid(W_g h) (mix.g [heads * vdim][width]) */
+  int qkv_bias;             /* 1: q, k, v = W h + b (mix.q.b, mix.k.b, mix.v.b) */
+  int qkv_conv;             /* > 0: taps of a causal convolution over time per channel of q, k, v right after the projection
+                               (mix.{q,k,v}.conv [channels][taps], no activation); its last taps - 1 inputs are state */
+  float score_softcap;      /* > 0: score <- cap * tanh(score / cap) */
+  int dist_bias;            /* 1: score <- score - r1[head] ln(1 + r2[head] (i - j)) (mix.r1, mix.r2) */
+  /* ---- TL_MIXER_DELTA ---- */
+  int decay_per_head;       /* 1: one decay per head, g = exp(-exp(A_log) softplus(W_a h + dt_bias)) with mix.a [heads][width]
+                               and dt_bias [heads] (decay_rank = 0); the output gate is silu(W_g h), mix.g [heads * vdim][width]
+                               (gate_rank = 0) */
+  /* ---- a second mixer beside the first, both reading the same input: the layer's mixer output is
+          mix_scale * mixer + side_scale * side. `side` is that mixer's entry (mixer fields only: block, feed-forward and
+          weights_of are the layer's). The first mixer's tensors are then l<i>.mix.left.*, the second's l<i>.mix.right.* ---- */
+  const struct tl_layer_spec* side;
+  float mix_scale, side_scale;
 } tl_layer_spec;
 typedef struct tl_stack_config {
   int width, vocab, n_layers;
@@ -345,6 +380,10 @@ typedef struct tl_stack_config {
   int norm;                 /* tl_norm_kind of the block norms and the final norm */
   int embed_norm;           /* 1: the embedding row is normalised (tensor embed.norm) before the first layer */
   float logit_softcap;      /* > 0: logits <- cap * tanh(logits / cap) */
+  float embed_scale;        /* != 0: the embedding row is multiplied by it */
+  int canon_taps;           /* > 0 (pre-norm blocks): what a sublayer reads is h + conv(h), a causal convolution over time per
+                               channel with so many taps (l<i>.canon1 for the mixer, l<i>.canon2 for the feed-forward,
+                               [width][taps], the last column is the current token's); the last taps - 1 inputs are state */
 } tl_stack_config;
 /* the operators such a model is built from, callable on their own (all FP32 in and out, weights bf16 [rows][cols]):
  * Y[T][rows] = X[T][cols] W^T; terms 1 / 3 = MFMA GEMM with bf16-rounded / three-term-split activations, 0 = FP32 GEMV (T = 1) */

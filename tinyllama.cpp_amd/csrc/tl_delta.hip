@@ -87,6 +87,11 @@ __global__ __launch_bounds__(128) void delta_pre_kernel(const DeltaPreArgs a) {
   const int h = unit - 2 * a.kv_heads, gd = a.heads * a.dim;
   if (tid == 0) a.beta[(size_t)t * a.heads + h] = sigmoidf_(a.p[(size_t)t * a.ld + C + h]);
   const float rate = expf(a.a_log[h]);
+  if (a.a_per_head) {  // one decay for the whole head, spread over its key channels
+    const float gh = expf(-rate * softplusf_(a.a[(size_t)t * a.a_ld + h] + a.dt_bias[h]));
+    for (int d = tid; d < a.dim; d += 128) a.g[(size_t)t * gd + h * a.dim + d] = gh;
+    return;
+  }
   for (int d = tid; d < a.dim; d += 128) {
     const int c = h * a.dim + d;
     a.g[(size_t)t * gd + c] = expf(-rate * softplusf_(a.a[(size_t)t * gd + c] + a.dt_bias[c]));
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const DeltaScanArgs a) 
     }
     const int tt = tid >> 4, c = blockIdx.x * 16 + (tid & 15);
     rv = (tt < DELTA_TB && t0 + tt < a.T && c < a.vdim) ? a.v[(size_t)(t0 + tt) * a.ldv + (size_t)h * a.vdim + c] : 0.0f;
-    rb = (tid < DELTA_TB && t0 + tid < a.T) ? a.beta[(size_t)(t0 + tid) * a.heads + h] : 0.0f;
+    rb = (tid < DELTA_TB && t0 + tid < a.T) ? (a.beta ? a.beta[(size_t)(t0 + tid) * a.heads + h] : 1.0f) : 0.0f;
   };
   auto stash = [&](int b) __attribute__((always_inline)) {
 #pragma unroll
@@ -193,7 +198,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const DeltaScanArgs a) 
       sk = row16_sum(sk);
       sq = row16_sum(sq);
       kq = row16_sum(kq);
-      const float u = bc * (vc - sk);
+      const float u = a.plain_write ? bc * vc : bc * (vc - sk);
 #pragma unroll
       for (int e = 0; e < E; ++e) s[e] += kc[e] * u;
       if (live && sub == 0) a.o[(size_t)(t0 + tt) * a.heads * a.vdim + (size_t)h * a.vdim + col] = sq + u * kq;
@@ -208,21 +213,40 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const DeltaScanArgs a) 
   }
 }
 
-// a wave per (token, head); gate rows gate_ld floats apart; w_stride = vdim: weights of its own for every head, 0: shared
-__global__ __launch_bounds__(256) void gated_head_norm_kernel(float* __restrict__ o, const float* __restrict__ gate, int gate_ld,
-                                                             const float* __restrict__ w, int w_stride, int heads,
-                                                             int n_heads_total, int vdim, float eps) {
+// a wave per (token, head); gate rows gate_ld floats apart; weights of its own for every head or one vector for all
+__global__ __launch_bounds__(256) void head_norm_kernel(const HeadNormArgs a) {
   const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (i >= n_heads_total) return;
-  const int t = i / heads, h = i - t * heads;
-  float* x = o + (size_t)i * vdim;
-  const float* g = gate + (size_t)t * gate_ld + (size_t)h * vdim;
-  const float* wh = w + (size_t)h * w_stride;
+  if (i >= a.T * a.heads) return;
+  const int t = i / a.heads, h = i - t * a.heads, vdim = a.vdim;
+  float* x = a.o + (size_t)i * vdim;
+  const float* sub = a.sub ? a.sub + (size_t)i * vdim : nullptr;
+  const float* g = a.gate ? a.gate + (size_t)t * a.gate_ld + (size_t)h * vdim : nullptr;
+  const float* wh = a.w ? a.w + (a.w_per_head ? (size_t)h * vdim : 0) : nullptr;
+  const float scale = a.out_scale != 0.0f ? a.out_scale : 1.0f;
   float ss = 0.0f;
-  for (int d = lane; d < vdim; d += 64) ss += x[d] * x[d];
+  for (int d = lane; d < vdim; d += 64) {
+    const float v = sub ? x[d] - a.sub_coef * sub[d] : x[d];
+    ss += v * v;
+  }
   ss = tl_wave_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
-  for (int d = lane; d < vdim; d += 64) x[d] = x[d] * inv * wh[d] * sigmoidf_(g[d]);
+  const float inv = 1.0f / sqrtf(ss / (float)vdim + a.eps);
+  for (int d = lane; d < vdim; d += 64) {
+    float v = (sub ? x[d] - a.sub_coef * sub[d] : x[d]) * inv * scale;
+    if (wh) v *= wh[d];
+    if (g) v *= a.gate_act == 1 ? g[d] * sigmoidf_(g[d]) : sigmoidf_(g[d]);
+    x[d] = v;
+  }
+}
+
+// grid (column blocks of 256 over heads * dim, T)
+__global__ __launch_bounds__(256) void linear_pre_kernel(const LinearPreArgs a) {
+  const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x, hd = a.heads * a.dim;
+  if (c >= hd) return;
+  const float* row = a.p + (size_t)t * a.ld;
+  const float q = row[c], z = row[hd + c] + a.f_bias[c], low = a.lower[c];
+  a.qk[(size_t)t * 2 * hd + c] = q * sigmoidf_(q);
+  a.qk[(size_t)t * 2 * hd + hd + c] = (1.0f - low) * sigmoidf_(-z);  // 1 - f
+  a.g[(size_t)t * hd + c] = low + (1.0f - low) * sigmoidf_(z);
 }
 
 // grid (T, heads): a workgroup of 128 threads owns one head of one token (dim <= 512: four channels a thread)
@@ -379,6 +403,7 @@ int tl_launch_delta_pre(const DeltaPreArgs& a, hipStream_t s) {
   TL_REQUIRE(a.taps >= 1 && (a.taps == 1 || a.hist), "delta_pre: %d taps", a.taps);
   const int C = 2 * a.kv_heads * a.dim + a.heads * a.vdim;
   TL_REQUIRE(a.ld >= C + a.heads, "delta_pre: row stride %d below %d", a.ld, C + a.heads);
+  TL_REQUIRE(!a.a_per_head || a.a_ld >= a.heads, "delta_pre: a decay per head with row stride %d", a.a_ld);
   TL_REQUIRE(a.dim <= 512 && a.vdim <= 512, "delta_pre: head sizes %d / %d above 512", a.dim, a.vdim);
   TL_REQUIRE(2 * a.kv_heads + a.heads <= 65535, "delta_pre: too many heads");
   delta_pre_kernel<<<dim3(a.T, 2 * a.kv_heads + a.heads), 128, 0, s>>>(a);
@@ -388,7 +413,7 @@ int tl_launch_delta_pre(const DeltaPreArgs& a, hipStream_t s) {
 }
 
 int tl_launch_delta_scan(const DeltaScanArgs& a, hipStream_t s) {
-  TL_REQUIRE(a.q && a.k && a.v && a.beta && a.g && a.state && a.o && a.T > 0, "delta_scan: bad arguments");
+  TL_REQUIRE(a.q && a.k && a.v && (a.beta || a.plain_write) && a.g && a.state && a.o && a.T > 0, "delta_scan: bad arguments");
   TL_REQUIRE(a.heads > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0 && a.dim > 0 && a.vdim > 0 && a.heads <= 65535,
              "delta_scan: %d heads over %d query/key heads, sizes %d / %d", a.heads, a.kv_heads, a.dim, a.vdim);
   TL_REQUIRE(a.dim <= 256, "delta_scan: key size %d above 256", a.dim);
@@ -405,10 +430,35 @@ int tl_launch_delta_scan(const DeltaScanArgs& a, hipStream_t s) {
 
 int tl_launch_gated_head_norm_rows(float* o, const float* gate, int gate_ld, const float* w, int w_per_head, int T, int heads,
                                    int vdim, float eps, hipStream_t s) {
-  TL_REQUIRE(o && gate && w && T > 0 && heads > 0 && vdim > 0 && gate_ld >= heads * vdim, "gated_head_norm: bad arguments");
-  const long long n = (long long)T * heads;
-  TL_REQUIRE(n <= 0x7fffffffLL, "gated_head_norm: too many heads");
-  gated_head_norm_kernel<<<(unsigned)((n + 3) / 4), 256, 0, s>>>(o, gate, gate_ld, w, w_per_head ? vdim : 0, heads, (int)n, vdim, eps);
+  TL_REQUIRE(o && gate && w, "gated_head_norm: bad arguments");
+  HeadNormArgs a = {};
+  a.o = o;
+  a.gate = gate;
+  a.gate_ld = gate_ld;
+  a.w = w;
+  a.w_per_head = w_per_head;
+  a.T = T;
+  a.heads = heads;
+  a.vdim = vdim;
+  a.eps = eps;
+  return tl_launch_head_norm(a, s);
+}
+
+int tl_launch_head_norm(const HeadNormArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.o && a.T > 0 && a.heads > 0 && a.vdim > 0 && (!a.gate || a.gate_ld >= a.heads * a.vdim), "head_norm: bad arguments");
+  TL_REQUIRE(a.gate_act == 0 || a.gate_act == 1, "head_norm: gate activation %d", a.gate_act);
+  const long long n = (long long)a.T * a.heads;
+  TL_REQUIRE(n <= 0x7fffffffLL, "head_norm: too many heads");
+  head_norm_kernel<<<(unsigned)((n + 3) / 4), 256, 0, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_linear_pre(const LinearPreArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.p && a.lower && a.f_bias && a.qk && a.g && a.T > 0 && a.T <= 65535 && a.heads > 0 && a.dim > 0,
+             "linear_pre: bad arguments");
+  TL_REQUIRE(a.ld >= 2 * a.heads * a.dim, "linear_pre: row stride %d below %d", a.ld, 2 * a.heads * a.dim);
+  linear_pre_kernel<<<dim3((a.heads * a.dim + 255) / 256, a.T), 256, 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
 #pragma unroll
           for (int e = 0; e < 2; ++e)
             if (f + 2 * e + 1 < a.rows)
-              yr[(f >> 1) + e] = dense_glu(acc[i][j][gq * 4 + 2 * e], acc[i][j][gq * 4 + 2 * e + 1], a.glu_limit, a.glu_alpha, a.glu_up_add);
+              yr[(f >> 1) + e] = tl_glu_apply(a.glu_kind, acc[i][j][gq * 4 + 2 * e], acc[i][j][gq * 4 + 2 * e + 1], a.glu_limit, a.glu_alpha, a.glu_up_add);
           continue;
         }
         if (a.softcap > 0.0f) {

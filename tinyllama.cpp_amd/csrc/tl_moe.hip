@@ -45,7 +45,10 @@ __global__ __launch_bounds__(1024) void router_kernel(const RouterArgs a, int ve
   }
   __syncthreads();
   if (wave != 0) return;
-  if (a.kind == TL_ROUTE_SOFTMAX_GROUPS)
+  if (a.kind == TL_ROUTE_SIGMOID_GROUPS)
+    tl_route_select_sigmoid_groups(z, z + a.experts, z + 2 * a.experts, a.corr, a.experts, a.top, a.groups, a.keep,
+                                   a.ids + (size_t)t * a.top, a.wts + (size_t)t * a.top, lane);
+  else if (a.kind == TL_ROUTE_SOFTMAX_GROUPS)
     tl_route_select_groups(z, z + a.experts, z + 2 * a.experts, a.experts, a.top, a.groups, a.keep, a.ids + (size_t)t * a.top,
                            a.wts + (size_t)t * a.top, lane);
   else
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(256) void moe_decode_gu_kernel(const MoeDecodeArgs 
   const unsigned short* gu = shared ? a.sgu : a.gu + (size_t)a.ids[j] * 2 * a.ff * a.width;
   float gu2[2];  // unit r's gate and up rows lie side by side; their loads are in flight together
   tl_wave_dot_rows<2>(gu + (size_t)2 * r * a.width, (size_t)a.width, 2, a.x, a.width, vec != 0, lane, gu2);
-  if (lane == 0) a.act[(size_t)j * a.ff + r] = glu_act(gu2[0], gu2[1], shared ? a.slimit : a.limit, a.alpha, a.up_add);
+  if (lane == 0) a.act[(size_t)j * a.ff + r] = tl_glu_apply(a.glu_kind, gu2[0], gu2[1], shared ? a.slimit : a.limit, a.alpha, a.up_add);
 }
 
 __global__ __launch_bounds__(256) void moe_decode_down_kernel(const MoeDecodeArgs a, int vec_e, int vec_s) {
@@ -123,7 +126,7 @@ int tl_launch_router(const RouterArgs& a, hipStream_t s) {
   TL_REQUIRE(a.top > 0 && a.top <= a.experts, "router: top %d of %d experts", a.top, a.experts);
   TL_REQUIRE(!a.gate_w || a.gate_out, "router: a gate row without an output");
   size_t lds = sizeof(float) * a.experts;
-  if (a.kind == TL_ROUTE_SOFTMAX_GROUPS) {
+  if (a.kind == TL_ROUTE_SOFTMAX_GROUPS || a.kind == TL_ROUTE_SIGMOID_GROUPS) {
     TL_REQUIRE(a.groups > 0 && a.experts % a.groups == 0 && a.keep > 0 && a.keep <= a.groups,
                "router: %d experts in %d groups, %d kept", a.experts, a.groups, a.keep);
     TL_REQUIRE((long long)a.keep * (a.experts / a.groups) >= a.top, "router: top %d of %d kept groups of %d", a.top, a.keep,
@@ -205,6 +208,25 @@ extern "C" int tl_moe_route_groups(const float* x_dev, int num_tokens, int width
   a.ids = ids_dev;
   a.wts = weights_dev;
   a.kind = TL_ROUTE_SOFTMAX_GROUPS;
+  a.groups = groups;
+  a.keep = keep;
+  return tl_launch_router(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tl_moe_route_sigmoid_groups(const float* x_dev, int num_tokens, int width, const void* w_bf16_dev,
+                                           const float* correction_dev, int experts, int top, int groups, int keep, int* ids_dev,
+                                           float* weights_dev, void* stream) {
+  RouterArgs a = {};
+  a.x = x_dev;
+  a.T = num_tokens;
+  a.width = width;
+  a.experts = experts;
+  a.top = top;
+  a.w = static_cast<const uint16_t*>(w_bf16_dev);
+  a.corr = correction_dev;
+  a.ids = ids_dev;
+  a.wts = weights_dev;
+  a.kind = TL_ROUTE_SIGMOID_GROUPS;
   a.groups = groups;
   a.keep = keep;
   return tl_launch_router(a, static_cast<hipStream_t>(stream));

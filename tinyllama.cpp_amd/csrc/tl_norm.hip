@@ -52,6 +52,25 @@ __global__ __launch_bounds__(1024) void qkv_post_kernel(const QkvPostArgs a) {
   float* q = a.qkv + (size_t)t * a.ld;
   const float* k = q + a.qd;
   const float* v = k + a.kd;
+  if (a.head_dim > 0) {  // every block of head_dim of q and of k on its own, one weight vector each: a wave per block in turn
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6, hd = a.head_dim;
+    const int nq = a.qd / hd, nk = a.kd / hd;
+    float* kr = a.kc + (size_t)pos * a.kd;
+    for (int g = wave; g < nq + nk; g += nw) {
+      const bool isq = g < nq;
+      const float* src = isq ? q + (size_t)g * hd : k + (size_t)(g - nq) * hd;
+      float* dst = isq ? q + (size_t)g * hd : kr + (size_t)(g - nq) * hd;
+      const float* w = isq ? a.q_norm : a.k_norm;
+      float ss = 0.0f;
+      for (int d = lane; d < hd; d += 64) ss += src[d] * src[d];
+      ss = tl_wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)hd + a.eps);
+      for (int d = lane; d < hd; d += 64) dst[d] = src[d] * inv * w[d];
+    }
+    float* vr = a.vc + (size_t)pos * a.vd;
+    for (int c = threadIdx.x; c < a.vd; c += blockDim.x) vr[c] = v[c];
+    return;
+  }
   float sq = 0.0f, sk = 0.0f;
   if (a.q_norm)
     for (int c = threadIdx.x; c < a.qd; c += blockDim.x) sq += q[c] * q[c];
@@ -126,7 +145,8 @@ __global__ __launch_bounds__(1024) void resid_norm_kernel(const ResidNormArgs a)
 }
 
 __global__ __launch_bounds__(1024) void norm_rows_kernel(const float* __restrict__ x, int width, const int* __restrict__ rows,
-                                                        const float* __restrict__ w, float eps, float* __restrict__ out) {
+                                                        const float* __restrict__ w, float eps, float* __restrict__ out,
+                                                        float w_add) {
   extern __shared__ __attribute__((aligned(16))) float row[];
   __shared__ float red[kMaxWaves];
   const int i = blockIdx.x;
@@ -139,7 +159,37 @@ __global__ __launch_bounds__(1024) void norm_rows_kernel(const float* __restrict
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  for (int c = threadIdx.x; c < width; c += blockDim.x) out[(size_t)i * width + c] = row[c] * inv * (1.0f + w[c]);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) out[(size_t)i * width + c] = row[c] * inv * (w_add + w[c]);
+}
+
+// pre-norm blocks with an RMS norm: the residual sum and the norm of what reads x next
+__global__ __launch_bounds__(1024) void resid_rms_kernel(const ResidRmsArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float row[];
+  __shared__ float red[kMaxWaves];
+  const int t = blockIdx.x;
+  float* xr = a.x + (size_t)t * a.width;
+  const bool add = a.a || a.b || a.slots;
+  float ss = 0.0f;
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+    float v = xr[c];
+    if (add) {
+      float y = a.a ? a.a_scale * a.a[(size_t)t * a.width + c] : 0.0f;
+      if (a.b) y += a.b_scale * a.b[(size_t)t * a.width + c];
+      if (a.slots) {
+        float e = 0.0f;
+        for (int j = 0; j < a.top; ++j) e += a.slot_w[t * a.top + j] * a.slots[((size_t)t * a.top + j) * a.width + c];
+        y += e;
+      }
+      v += y;
+      xr[c] = v;
+    }
+    row[c] = v;
+    ss += v * v;
+  }
+  if (!a.w) return;
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)a.width + a.eps), w_add = a.one_plus ? 1.0f : 0.0f;
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) a.h[(size_t)t * a.width + c] = row[c] * inv * (w_add + a.w[c]);
 }
 
 constexpr int kMaxRowFloats = 16 * 1024;  // 64 KB of LDS for the staged row
@@ -218,11 +268,11 @@ __device__ __forceinline__ float dyt_of(float x, float alpha, float w, float b) 
 // grid (column blocks of 256, T)
 __global__ __launch_bounds__(256) void embed_rows_kernel(const unsigned short* __restrict__ table, int vocab, int width,
                                                         const int* __restrict__ tokens, float* __restrict__ x,
-                                                        const DytParams next, float* __restrict__ h) {
+                                                        const DytParams next, float* __restrict__ h, float scale) {
   const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
   if (c >= width) return;
   const int tok = tokens[t];
-  const float v = (tok >= 0 && tok < vocab) ? __uint_as_float((unsigned)table[(size_t)tok * width + c] << 16) : 0.0f;
+  const float v = (tok >= 0 && tok < vocab) ? __uint_as_float((unsigned)table[(size_t)tok * width + c] << 16) * scale : 0.0f;
   x[(size_t)t * width + c] = v;
   if (next.alpha) h[(size_t)t * width + c] = dyt_of(v, *next.alpha, next.w[c], next.b[c]);
 }
@@ -253,10 +303,10 @@ __global__ __launch_bounds__(256) void dyt_rows_kernel(const float* __restrict__
 }  // namespace
 
 int tl_launch_embed_rows(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, float* x, const DytParams& next,
-                         float* h, hipStream_t s) {
+                         float* h, hipStream_t s, float scale) {
   TL_REQUIRE(table && tokens_dev && x && T > 0 && T <= 65535 && vocab > 0 && width > 0, "embed_rows: bad arguments");
   TL_REQUIRE(!next.alpha || (next.w && next.b && h), "embed_rows: a norm without its weights or output");
-  embed_rows_kernel<<<dim3((width + 255) / 256, T), 256, 0, s>>>(table, vocab, width, tokens_dev, x, next, h);
+  embed_rows_kernel<<<dim3((width + 255) / 256, T), 256, 0, s>>>(table, vocab, width, tokens_dev, x, next, h, scale);
   TL_HIP(hipGetLastError());
   return 0;
 }
@@ -331,6 +381,9 @@ int tl_launch_qkv_post(const QkvPostArgs& a, hipStream_t s) {
              "qkv_post: bad arguments");
   TL_REQUIRE(a.vmix == 0 || a.v_first, "qkv_post: value mixing without a v_first buffer");
   TL_REQUIRE(a.vmix != 2 || a.lambda, "qkv_post: value mixing without its coefficient");
+  TL_REQUIRE(a.head_dim == 0 || (a.head_dim > 0 && a.qd % a.head_dim == 0 && a.kd % a.head_dim == 0 && a.q_norm && a.k_norm &&
+                                 a.vmix == 0 && a.q_temp_every == 0),
+             "qkv_post: a norm per block of %d over %d / %d", a.head_dim, a.qd, a.kd);
   qkv_post_kernel<<<a.T, row_threads(a.T), 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
@@ -352,11 +405,21 @@ int tl_launch_resid_norm(const ResidNormArgs& a, hipStream_t s) {
   return 0;
 }
 
+int tl_launch_resid_rms(const ResidRmsArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.x && a.T > 0 && (a.w || a.a || a.b || a.slots), "resid_rms: bad arguments");
+  TL_REQUIRE(a.width > 0 && a.width <= kMaxRowFloats, "resid_rms: width %d outside (0, %d]", a.width, kMaxRowFloats);
+  TL_REQUIRE(!a.slots || (a.slot_w && a.top > 0), "resid_rms: expert slots without weights");
+  TL_REQUIRE(!a.w || a.h, "resid_rms: a norm without its output");
+  resid_rms_kernel<<<a.T, row_threads(a.T), sizeof(float) * a.width, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
 int tl_launch_norm_rows(const float* x, int width, const int* rows_dev, int n, const float* w, float eps, float* out,
-                        hipStream_t s) {
+                        hipStream_t s, int one_plus) {
   TL_REQUIRE(x && w && out && n > 0, "norm_rows: bad arguments");
   TL_REQUIRE(width > 0 && width <= kMaxRowFloats, "norm_rows: width %d outside (0, %d]", width, kMaxRowFloats);
-  norm_rows_kernel<<<n, row_threads(n), sizeof(float) * width, s>>>(x, width, rows_dev, w, eps, out);
+  norm_rows_kernel<<<n, row_threads(n), sizeof(float) * width, s>>>(x, width, rows_dev, w, eps, out, one_plus ? 1.0f : 0.0f);
   TL_HIP(hipGetLastError());
   return 0;
 }

@@ -145,3 +145,92 @@ __device__ __forceinline__ void tl_route_select_groups(float* z, float* key, flo
   }
   for (int j = lane; j < top; j += 64) wts[j] = wts[j] / (denom + 1e-20f);
 }
+
+// One wave: scores = sigmoid(z) (left in z[]); choice = score + corr[expert] (corr may be NULL); the experts form `groups` equal
+// groups of neighbours, a group ranks by the sum of its two best choices (its one choice when a group is one expert), and only
+// experts of the best `keep` groups (lower index among equals) can be chosen -- the others count as minus infinity, since a
+// choice may be negative; ids[top] = the best choices first (lower index among equals); wts = the chosen experts' SCORES,
+// without the correction and not normalised. key[experts] and gs[groups] are LDS scratch.
+__device__ __forceinline__ void tl_route_select_sigmoid_groups(float* z, float* key, float* gs, const float* corr, int experts,
+                                                               int top, int groups, int keep, int* ids, float* wts, int lane) {
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  const int per = experts / groups;
+  for (int e = lane; e < experts; e += 64) {
+    const float sc = 1.0f / (1.0f + expf(-z[e]));
+    z[e] = sc;
+    key[e] = sc + (corr ? corr[e] : 0.0f);
+  }
+  wave_sync();
+  for (int g = lane; g < groups; g += 64) {
+    float b1 = -INFINITY, b2 = -INFINITY;
+    for (int e = g * per; e < (g + 1) * per; ++e) {
+      const float v = key[e];
+      if (v > b1) {
+        b2 = b1;
+        b1 = v;
+      } else if (v > b2) {
+        b2 = v;
+      }
+    }
+    gs[g] = per > 1 ? b1 + b2 : b1;
+  }
+  wave_sync();
+  // groups are ranked `keep` times; a kept group is marked by +infinity in gs, the rest lose their choices afterwards
+  for (int r = 0; r < keep; ++r) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int g = lane; g < groups; g += 64) {
+      const float v = gs[g];
+      if (v != INFINITY && (v > bv || (v == bv && g < bi) || bi == 0x7fffffff)) {
+        bv = v;
+        bi = g;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(bv, o);
+      const int oi = __shfl_xor(bi, o);
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi == 0x7fffffff) bi = 0;
+    if (lane == 0) gs[bi] = INFINITY;
+    wave_sync();
+  }
+  for (int e = lane; e < experts; e += 64)
+    if (gs[e / per] != INFINITY) key[e] = -INFINITY;
+  wave_sync();
+  for (int j = 0; j < top; ++j) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < experts; e += 64) {
+      const float v = key[e];
+      if (v > bv || (v == bv && e < bi)) {
+        bv = v;
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(bv, o);
+      const int oi = __shfl_xor(bi, o);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi == 0x7fffffff) bi = 0;
+    if (lane == 0) {
+      ids[j] = bi;
+      wts[j] = z[bi];
+      key[bi] = -INFINITY;
+    }
+    wave_sync();
+  }
+}

@@ -35,6 +35,7 @@ struct DenseArgs {
   int glu;
   float glu_limit, glu_alpha;
   float glu_up_add;      // 1 in the formula above; a design may add something else (0: the plain gated unit)
+  int glu_kind;          // tl_glu_kind (0: the clamped swish unit above; TL_GLU_RELU: max(gate, 0) * up)
   float softcap;         // > 0 (not with glu): y <- softcap * tanh(y / softcap)
   // act != 0 (not with glu): a tl_act_kind on the output features from act_from on (TL_ACT_XIELU: act_p = softplus(p),
   // act_q = 1/2 + softplus(q))
@@ -60,6 +61,14 @@ __host__ __device__ inline float tl_act_apply(int act, float z, float p, float q
   if (act == TL_ACT_XIELU) return z > 0.0f ? p * z * z + 0.5f * z : q * (expm1f(z) - z) + 0.5f * z;
   if (act == TL_ACT_TANH) return tanhf(z);
   return z;
+}
+
+// the gated unit of tl_glu_kind, for every kernel that applies it
+__host__ __device__ inline float tl_glu_apply(int kind, float g, float u, float limit, float alpha, float up_add) {
+  if (kind == TL_GLU_RELU) return fmaxf(g, 0.0f) * u;
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + up_add);
 }
 
 // ---- tl_swa.hip --------------------------------------------------------------------------------------------------------
@@ -92,6 +101,13 @@ struct SwaArgs {
   // rows of the caches are kld / vld floats apart (0: kv_heads * dim, kv_heads * vdim): a cache of latent rows serves as
   // keys (the whole row) and values (its first vdim columns) at once
   int kld, vld;
+  // heads of a query row / key row are q_hstride / k_hstride floats apart (0: dim): with two score maps per head laid out side
+  // by side, one launch per map walks every second block of dim
+  int q_hstride, k_hstride;
+  float softcap;            // > 0: score <- softcap * tanh(score / softcap), after the scale
+  const float* dist_r1;     // optional [heads] (with dist_r2): score <- score - r1 ln(1 + r2 (i - j)), after the cap
+  const float* dist_r2;
+  const float* sink_val;    // with sink: the sink's score per head (NULL: 0)
 };
 int tl_launch_swa(const SwaArgs& a, hipStream_t s);
 int tl_swa_splits(int T, int window, int max_pos, int keep_first = 0);  // splits worth having for T tokens over a cache of max_pos rows
@@ -117,6 +133,9 @@ struct QkvPostArgs {
   // q_temp_every > 0: q at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)
   float q_temp_coef;
   int q_temp_every;
+  // head_dim > 0: q_norm / k_norm are ONE weight vector [head_dim] each and every block of head_dim of q and of k is
+  // RMS-normed on its own (per head, and per score map where a head has several)
+  int head_dim;
 };
 int tl_launch_qkv_post(const QkvPostArgs& a, hipStream_t s);
 // (declared here because the residual norm may carry it; the launcher is tl_moe.hip's)
@@ -133,6 +152,9 @@ struct RouterArgs {
   // optional: one more row of weights whose logit becomes a gate per token, gate_out[t] = sigmoid(gate_w . x[t])
   const uint16_t* gate_w;
   float* gate_out;
+  // kind = TL_ROUTE_SIGMOID_GROUPS: scores = sigmoid(logits), choice = score + corr[expert]; a group ranks by the sum of its two
+  // best choices; wts = the chosen experts' scores as they are
+  const float* corr;
 };
 struct ResidNormArgs {
   float* x;              // [T][width] residual stream, updated in place: x += y / rms(y) * (1 + w)
@@ -148,6 +170,24 @@ struct ResidNormArgs {
   RouterArgs route;
 };
 int tl_launch_resid_norm(const ResidNormArgs& a, hipStream_t s);
+// pre-norm blocks with an RMS norm: x[t] += a_scale a[t] + b_scale b[t] + sum_j slot_w[j] slots[j]; then, when w is set,
+// h[t] = x[t] / sqrt(mean(x[t]^2) + eps) * w (one_plus: * (1 + w)): the norm in front of the sublayer that reads x next
+struct ResidRmsArgs {
+  float* x;              // [T][width]
+  int T, width;
+  const float* a;        // optional [T][width]
+  float a_scale;
+  const float* b;        // optional [T][width]
+  float b_scale;
+  const float* slots;    // optional [T * top][width] expert outputs, weighted by slot_w
+  const float* slot_w;   // [T * top]
+  int top;
+  const float* w;        // [width] (NULL: no norm asked for)
+  int one_plus;
+  float eps;
+  float* h;              // [T][width]
+};
+int tl_launch_resid_rms(const ResidRmsArgs& a, hipStream_t s);
 // ---- norm-first blocks: Dynamic Tanh (elementwise, no statistics) and the plain residual sum ------------------------------
 struct DytParams {
   const float* alpha;    // device scalar (NULL: no norm asked for)
@@ -156,7 +196,7 @@ struct DytParams {
 };
 // x[t] = embed[token[t]] (an id outside the table embeds as zeros); h[t] = tanh(alpha x[t]) * w + b when next.alpha is set
 int tl_launch_embed_rows(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, float* x, const DytParams& next,
-                         float* h, hipStream_t s);
+                         float* h, hipStream_t s, float scale = 1.0f);
 struct ResidSumArgs {
   float* x;              // [T][width] residual stream: x += a + b * b_gate + sum_j slot_w[j] slots[j]
   int T, width;
@@ -174,7 +214,7 @@ int tl_launch_resid_sum(const ResidSumArgs& a, hipStream_t s);
 int tl_launch_dyt_rows(const float* x, int width, const int* rows_dev, int n, const DytParams& p, float* out, hipStream_t s);
 // out[i] = x[rows[i]] / rms * (1 + w)   (rows == NULL: row i)
 int tl_launch_norm_rows(const float* x, int width, const int* rows_dev, int n, const float* w, float eps, float* out,
-                        hipStream_t s);
+                        hipStream_t s, int one_plus = 1);
 
 // ---- layer norm (pre-norm blocks): (x - mean) / sqrt(var + eps) * w + b, statistics in FP32 over the row staged in LDS -------
 struct LnParams {
@@ -189,6 +229,23 @@ int tl_launch_resid_ln(float* x, const float* a, int T, int width, const LnParam
 // out[i] = ln(x[rows[i]]; p)   (rows == NULL: row i)
 int tl_launch_ln_rows(const float* x, int width, const int* rows_dev, int n, const LnParams& p, float eps, float* out,
                       hipStream_t s);
+
+// ---- tl_conv.hip: a short causal convolution over time per channel, with its history as state ----------------------------
+// out[t][c] = act(sum_j w[c][j] u[t - taps + 1 + j][c]) (+ u[t][c] with add_input), u[t][c] = in[t][c] (+ bias[c]); the inputs
+// of the taps - 1 tokens before this call come from hist [taps - 1][C] (oldest first; zeros for an empty sequence), which
+// afterwards holds the last taps - 1 inputs u. out must not overlap in when T > 1.
+struct ConvArgs {
+  const float* in;       // [T][ldi], channels [0, C)
+  int ldi, C, taps, T;
+  const float* bias;     // optional [C]
+  const uint16_t* w;     // bf16 [C][taps], the last tap is the current token's
+  float* hist;           // [taps - 1][C]
+  int act;               // 0: none, 1: silu
+  int add_input;
+  float* out;            // [T][ldo]
+  int ldo;
+};
+int tl_launch_causal_conv(const ConvArgs& a, hipStream_t s);
 
 // ---- tl_latent.hip: what sits between the products of a latent-attention mixer ------------------------------------------
 struct LatentPostArgs {
@@ -248,6 +305,7 @@ struct MoeDecodeArgs {
   float* y;              // [width]
   float up_add;          // the gated unit's (u + up_add)
   const float* sgate;    // optional device scalar: factor on the shared expert's output
+  int glu_kind;          // tl_glu_kind
 };
 int tl_launch_moe_decode(const MoeDecodeArgs& a, hipStream_t s);
 
@@ -292,6 +350,9 @@ struct DeltaPreArgs {
   float* qkv;            // out [T][channels]: silu(conv), q and k unit vectors per head (eps 1e-6), q times dim^-1/2
   float* beta;           // out [T][heads] = sigmoid
   float* g;              // out [T][heads * dim] = exp(-exp(a_log) softplus(a + dt_bias))
+  // a_per_head != 0: one decay per head -- a holds one pre-activation per head (token t, head h at a + t * a_ld + h), dt_bias
+  // is [heads], and g receives the head's decay in every key channel
+  int a_per_head, a_ld;
 };
 int tl_launch_delta_pre(const DeltaPreArgs& a, hipStream_t s);
 struct DeltaScanArgs {
@@ -305,6 +366,9 @@ struct DeltaScanArgs {
   float* state;          // [heads][vdim][dim]: column c of head h's S, contiguous over the key channels; updated
   float* o;              // [T][heads * vdim]
   int T, heads, kv_heads, dim, vdim;
+  // plain_write != 0: nothing is removed before the write, u = beta v (a gated linear recurrence S <- diag(g) S + k v^T);
+  // beta may then be NULL (1)
+  int plain_write;
 };
 int tl_launch_delta_scan(const DeltaScanArgs& a, hipStream_t s);
 // o[t][h] <- o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t][h]) per head (w [vdim] shared by the heads); in place
@@ -312,6 +376,32 @@ int tl_launch_gated_head_norm(float* o, const float* gate, const float* w, int T
 // the same with gate rows gate_ld floats apart and, w_per_head != 0, weights [heads * vdim] of their own for every head
 int tl_launch_gated_head_norm_rows(float* o, const float* gate, int gate_ld, const float* w, int w_per_head, int T, int heads,
                                    int vdim, float eps, hipStream_t s);
+// the general form: o <- (o - sub_coef * sub) / sqrt(mean(.^2) + eps) * w * gate_fn(gate) * out_scale per head; sub, w and gate
+// are optional; gate_act 0: sigmoid, 1: silu
+struct HeadNormArgs {
+  float* o;              // [T][heads * vdim], in place
+  const float* sub;      // optional [T][heads * vdim]
+  float sub_coef;
+  const float* gate;     // optional, token t at gate + t * gate_ld
+  int gate_ld, gate_act;
+  const float* w;        // optional [vdim] (w_per_head: [heads * vdim])
+  int w_per_head;
+  float out_scale;       // 0: 1
+  int T, heads, vdim;
+  float eps;
+};
+int tl_launch_head_norm(const HeadNormArgs& a, hipStream_t s);
+// what precedes the gated linear recurrence of TL_MIXER_LINEAR: p [T][ld] = q | f (heads * dim each) | ...;
+// qk [T][2 * heads * dim] = silu(q) | 1 - f, g [T][heads * dim] = f, f = lower + (1 - lower) sigmoid(p_f + f_bias)
+struct LinearPreArgs {
+  const float* p;
+  int ld, T, heads, dim;
+  const float* lower;    // [heads * dim]
+  const float* f_bias;   // [heads * dim]
+  float* qk;
+  float* g;
+};
+int tl_launch_linear_pre(const LinearPreArgs& a, hipStream_t s);
 // ---- generalized delta rule: S <- diag(w) S - (a u)(u^T S) + k v^T (both terms read the old S), o = S^T r ------------------
 struct GDeltaPreArgs {
   const float* p;        // [T][ld]: r | k | v | gate | a, heads * dim each (the gate is not read here)

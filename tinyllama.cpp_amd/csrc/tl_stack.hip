@@ -38,6 +38,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <memory>
 #include <set>
 #include <string>
 #include <vector>
@@ -77,6 +78,15 @@ struct Layer {
   // generalized delta rule: wqkv = r | k | v | g | a | w1 stacked, wa2 = w2
   float *w0 = nullptr, *a_bias = nullptr;
   float act_p = 0.0f, act_q = 0.0f;          // TL_MLP_UNIT: the activation's two numbers, transformed (tl_act_kind)
+  // windowed attention with its options: biases of q | k | v, a convolution on them (conv, hist above), distance bias, sink
+  // scores per head; two score maps: lambda from four vectors kept on the host until all have arrived
+  float *qkv_b = nullptr, *r1 = nullptr, *r2 = nullptr, *sinkv = nullptr;
+  std::vector<float> lvec[4];
+  float lam = 0.0f;
+  float *lower = nullptr, *f_bias = nullptr;  // gated linear attention: lower bound and bias of the forget gate
+  uint16_t *canon1 = nullptr, *canon2 = nullptr;          // convolutions on what the sublayers read [width][taps]
+  float *canon_hist1 = nullptr, *canon_hist2 = nullptr;   // ... and their last taps - 1 inputs (state)
+  std::unique_ptr<Layer> side;               // the second mixer of a pair: its mixer fields, tensors and state only
   std::set<std::string> expect, optional;    // tensor names (without the "l<i>." prefix) still missing / accepted and ignored
 };
 
@@ -107,6 +117,9 @@ struct TlStack {
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   // workspaces for one chunk
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *proj = nullptr, *v_first = nullptr, *xn = nullptr;
+  float *att2 = nullptr, *proj2 = nullptr;  // the second score map of differential attention; the second mixer of a pair
+  float* hn = nullptr;      // the norm of x before the convolution on what a sublayer reads
+  bool any_pair = false, any_maps = false;
   float* h = nullptr;       // norm-first blocks: the normalised input both sublayers read
   float *dq = nullptr, *da = nullptr, *dg = nullptr, *dbeta = nullptr, *ddecay = nullptr;  // delta rule
   float *lq = nullptr, *lqa = nullptr;      // latent attention: up-projected queries, absorbed queries
@@ -179,12 +192,376 @@ bool shape_is(const long long* shape, int ndim, long long a, long long b = -1) {
 
 }  // namespace
 
+namespace {
+
+int upload_frequencies(TlStack* st, Layer& L, const std::vector<double>& f) {
+  TL_TRY(dev_alloc(st, &L.freq, f.size()));
+  TL_HIP(hipMemcpy(L.freq, f.data(), sizeof(double) * f.size(), hipMemcpyHostToDevice));
+  return 0;
+}
+
+// The mixer of layer i (or the second mixer of its pair): checks, sizes, tensor names, device buffers of its tensors (own:
+// the layer holds tensors of its own) and its share of the cache. first_mix: the first value-mixing layer so far.
+int setup_mixer(TlStack* st, Layer& L, int i, bool own, int* first_mix) {
+  const tl_stack_config* cfg = &st->cfg;
+  const tl_layer_spec& sp = L.sp;
+  const size_t W = cfg->width;
+  TL_REQUIRE(sp.mixer >= TL_MIXER_SWA && sp.mixer <= TL_MIXER_LINEAR,
+             "tl_stack_create: layer %d has mixer kind %d; this engine has windowed attention (%d), the gated delta rule (%d), "
+             "latent attention (%d), the generalized delta rule (%d) and gated linear attention (%d)",
+             i, sp.mixer, TL_MIXER_SWA, TL_MIXER_DELTA, TL_MIXER_LATENT, TL_MIXER_GDELTA, TL_MIXER_LINEAR);
+  TL_REQUIRE(sp.heads > 0 && sp.kv_heads > 0 && sp.heads % sp.kv_heads == 0 && sp.dim > 0 && sp.vdim > 0,
+             "tl_stack_create: layer %d: %d heads / %d key-value heads / sizes %d, %d", i, sp.heads, sp.kv_heads, sp.dim, sp.vdim);
+  if (sp.mixer == TL_MIXER_SWA) {
+    TL_REQUIRE(!sp.values_are_keys || sp.vdim == sp.dim, "tl_stack_create: layer %d: values that are keys need vdim == dim", i);
+    TL_REQUIRE(sp.rot_dims >= 0 && sp.rot_dims <= sp.dim && (sp.rot_dims & 1) == 0 && (sp.rot_dims == 0 || sp.rot_base > 0.0f),
+               "tl_stack_create: layer %d: %d rotating dimensions of %d, base %g", i, sp.rot_dims, sp.dim, sp.rot_base);
+    TL_REQUIRE(sp.keep_first >= 0, "tl_stack_create: layer %d: %d kept first keys", i, sp.keep_first);
+    TL_REQUIRE(sp.attn_weight >= TL_ATTN_SOFTMAX && sp.attn_weight <= TL_ATTN_SOFTMAX_LEARNED_SINK && sp.q_temp_every >= 0,
+               "tl_stack_create: layer %d: attention weights of kind %d, query temperature every %d", i, sp.attn_weight,
+               sp.q_temp_every);
+    L.rotary_path = sp.rot_dims > 0 || sp.qk_norm == TL_QK_NORM_HEAD_UNIT || sp.values_are_keys;
+    TL_REQUIRE(!L.rotary_path || (sp.qk_norm != TL_QK_NORM_WHOLE && sp.qk_norm != TL_QK_NORM_HEAD_RMS && !sp.v_mix &&
+                                  sp.q_temp_every == 0 && sp.score_maps <= 1 && !sp.qkv_conv && !sp.qkv_bias),
+               "tl_stack_create: layer %d: rotation / per-head unit norm / values-are-keys do not combine with the weighted q/k "
+               "norms, value mixing, a query temperature, score maps or a convolution on q, k, v", i);
+    TL_REQUIRE(sp.qk_norm >= TL_QK_NORM_NONE && sp.qk_norm <= TL_QK_NORM_HEAD_RMS, "tl_stack_create: layer %d: q/k norm %d", i, sp.qk_norm);
+    TL_REQUIRE(sp.score_maps == 0 || sp.score_maps == 1 || sp.score_maps == 2, "tl_stack_create: layer %d: %d score maps", i, sp.score_maps);
+    const int maps = sp.score_maps == 2 ? 2 : 1;
+    TL_REQUIRE(maps == 1 || (sp.attn_weight == TL_ATTN_SOFTMAX && !sp.v_mix && sp.q_temp_every == 0 && sp.keep_first == 0),
+               "tl_stack_create: layer %d: two score maps take the plain softmax", i);
+    TL_REQUIRE(!sp.out_gate || maps == 2, "tl_stack_create: layer %d: the output gate rides in the combination of two score maps", i);
+    TL_REQUIRE(sp.qk_norm != TL_QK_NORM_HEAD_RMS || (!sp.v_mix && sp.q_temp_every == 0),
+               "tl_stack_create: layer %d: the per-head q/k norm does not combine with value mixing or a query temperature", i);
+    TL_REQUIRE(sp.qkv_conv >= 0 && sp.qkv_conv <= 64 && (!sp.qkv_bias || sp.qkv_conv > 0) && (!sp.qkv_conv || !sp.v_mix),
+               "tl_stack_create: layer %d: %d taps on q, k, v (biases ride in that convolution)", i, sp.qkv_conv);
+    TL_REQUIRE(sp.score_softcap >= 0.0f, "tl_stack_create: layer %d: score cap %g", i, sp.score_softcap);
+    L.qd = sp.heads * sp.dim * maps;
+    L.kd = sp.kv_heads * sp.dim * maps;
+    L.vd = sp.kv_heads * sp.vdim;
+    L.od = sp.heads * sp.vdim;
+    L.gate_off = L.qd + L.kd + (sp.values_are_keys ? 0 : L.vd);
+    L.pd = L.gate_off + (sp.out_gate ? L.od : 0);
+    if (maps == 2) st->any_maps = true;
+    if (sp.v_mix) {
+      if (*first_mix < 0) {
+        *first_mix = i;
+        L.vmix_mode = 1;
+      } else {
+        L.vmix_mode = 2;
+        TL_REQUIRE(st->layers[*first_mix].vd == L.vd, "tl_stack_create: layer %d mixes %d values with the %d of layer %d", i,
+                   L.vd, st->layers[*first_mix].vd, *first_mix);
+      }
+    }
+    st->cache_bytes += sizeof(float) * (size_t)cfg->max_positions * (L.kd + L.vd);
+    if (sp.qkv_conv > 0) {
+      const int dc = L.qd + L.kd + L.vd;
+      st->max_dc = dc > st->max_dc ? dc : st->max_dc;
+      st->cache_bytes += sizeof(float) * (size_t)(sp.qkv_conv - 1) * dc;
+    }
+    if (own) {
+      L.expect.insert({"mix.q", "mix.k", "mix.o"});
+      if (!sp.values_are_keys) L.expect.insert("mix.v");
+      if (sp.qk_norm == TL_QK_NORM_WHOLE || sp.qk_norm == TL_QK_NORM_HEAD_RMS) L.expect.insert({"mix.q.norm", "mix.k.norm"});
+      else L.optional.insert({"mix.q.norm", "mix.k.norm"});
+      if (L.vmix_mode == 2) L.expect.insert("mix.vmix");
+      else L.optional.insert("mix.vmix");
+      if (sp.attn_weight == TL_ATTN_SIGMOID) L.expect.insert("mix.pb");
+      if (sp.attn_weight == TL_ATTN_SOFTMAX_LEARNED_SINK) L.expect.insert("mix.sink");
+      if (maps == 2) L.expect.insert({"mix.lq1", "mix.lk1", "mix.lq2", "mix.lk2"});
+      if (sp.out_gate) L.expect.insert("mix.g");
+      if (sp.qkv_bias) L.expect.insert({"mix.q.b", "mix.k.b", "mix.v.b"});
+      if (sp.qkv_conv > 0) L.expect.insert({"mix.q.conv", "mix.k.conv", "mix.v.conv"});
+      if (sp.dist_bias) L.expect.insert({"mix.r1", "mix.r2"});
+      TL_TRY(dev_alloc(st, &L.q_norm, L.qd));
+      TL_TRY(dev_alloc(st, &L.k_norm, L.kd));
+      TL_TRY(dev_alloc(st, &L.lambda, 1));
+      TL_TRY(dev_alloc(st, &L.pb, sp.heads));
+      TL_TRY(dev_alloc(st, &L.sinkv, sp.heads));
+      TL_TRY(dev_alloc(st, &L.r1, sp.heads));
+      TL_TRY(dev_alloc(st, &L.r2, sp.heads));
+      if (sp.qkv_bias) TL_TRY(dev_alloc(st, &L.qkv_b, (size_t)L.qd + L.kd + L.vd));
+      if (sp.qkv_conv > 0) TL_TRY(dev_alloc(st, &L.conv, (size_t)(L.qd + L.kd + L.vd) * sp.qkv_conv));
+      if (sp.rot_dims > 0) {
+        std::vector<double> f(sp.rot_dims / 2);
+        tl_rotary_frequencies(sp.rot_dims, sp.rot_base, sp.rot_factor, sp.rot_original, sp.rot_fast, sp.rot_slow, f.data(), &L.mscale);
+        TL_TRY(upload_frequencies(st, L, f));
+      }
+    }
+  } else if (sp.mixer == TL_MIXER_LATENT) {
+    TL_REQUIRE(sp.q_rank > 0 && sp.kv_rank > 0 && sp.rot_dim >= 0 && sp.rot_dims >= 0 && sp.rot_dims <= sp.rot_dim &&
+                   (sp.rot_dims & 1) == 0 && (sp.rot_dims == 0 || sp.rot_base > 0.0f) && sp.kv_heads == sp.heads,
+               "tl_stack_create: layer %d: latents of %d / %d, %d rotated dimensions of which %d turn (base %g), %d key heads",
+               i, sp.q_rank, sp.kv_rank, sp.rot_dim, sp.rot_dims, sp.rot_base, sp.kv_heads);
+    TL_REQUIRE(sp.kv_rank <= 512, "tl_stack_create: layer %d: a key/value latent of %d above 512", i, sp.kv_rank);
+    TL_REQUIRE(sp.weights_of == 0 && own, "tl_stack_create: layer %d: a latent layer owns its tensors (it may share a cache: kv_from)", i);
+    L.kv_src = i;
+    if (sp.kv_from > 0) {
+      const int j = sp.kv_from - 1;
+      TL_REQUIRE(j < i && st->layers[j].sp.mixer == TL_MIXER_LATENT && st->layers[j].sp.kv_from == 0,
+                 "tl_stack_create: layer %d reads the latent cache of layer %d, which is not an earlier latent layer "
+                 "with a projection of its own", i, j);
+      const tl_layer_spec& o = st->layers[j].sp;
+      TL_REQUIRE(o.kv_rank == sp.kv_rank && o.rot_dim == sp.rot_dim && o.rot_dims == sp.rot_dims && o.rot_base == sp.rot_base,
+                 "tl_stack_create: layer %d and layer %d, whose latent cache it reads, differ in latent size or rotation", i, j);
+      L.kv_src = j;
+    }
+    const bool own_kv = L.kv_src == i;
+    const int qh = sp.dim + sp.rot_dim, ah = sp.kv_rank + sp.rot_dim;
+    L.qd = sp.heads * qh;
+    L.kd = own_kv ? sp.kv_rank + sp.rot_dim : 0;
+    L.vd = 0;
+    L.od = sp.heads * sp.vdim;
+    L.gate_off = sp.q_rank + L.kd;
+    L.pd = L.gate_off + (sp.head_gate ? sp.heads : 0);
+    if (own_kv) st->cache_bytes += sizeof(float) * (size_t)cfg->max_positions * L.kd;
+    st->max_lq = L.qd > st->max_lq ? L.qd : st->max_lq;
+    st->max_lqa = sp.heads * ah > st->max_lqa ? sp.heads * ah : st->max_lqa;
+    st->max_lk = sp.heads * qh > st->max_lk ? sp.heads * qh : st->max_lk;
+    st->max_lv = sp.heads * sp.vdim > st->max_lv ? sp.heads * sp.vdim : st->max_lv;
+    st->max_od = sp.heads * sp.kv_rank > st->max_od ? sp.heads * sp.kv_rank : st->max_od;  // the weighted latents of all heads
+    L.expect.insert({"mix.dq", "mix.dq.norm", "mix.uq", "mix.uk", "mix.uv", "mix.o"});
+    if (own_kv) L.expect.insert({"mix.dkv", "mix.dkv.norm"});
+    if (sp.head_gate) L.expect.insert("mix.g");
+    TL_TRY(dev_alloc(st, &L.wuq, (size_t)L.qd * sp.q_rank));
+    TL_TRY(dev_alloc(st, &L.wukt, (size_t)sp.heads * sp.kv_rank * sp.dim));
+    TL_TRY(dev_alloc(st, &L.wuk, (size_t)sp.heads * sp.kv_rank * sp.dim));
+    TL_TRY(dev_alloc(st, &L.wuv, (size_t)sp.heads * sp.vdim * sp.kv_rank));
+    TL_TRY(dev_alloc(st, &L.dq_norm, sp.q_rank));
+    TL_TRY(dev_alloc(st, &L.dkv_norm, sp.kv_rank));
+    if (sp.rot_dims > 0) {
+      std::vector<double> f(sp.rot_dims / 2);
+      float unused = 1.0f;
+      tl_rotary_frequencies(sp.rot_dims, sp.rot_base, 0.0, 0.0, 0.0, 0.0, f.data(), &unused);
+      TL_TRY(upload_frequencies(st, L, f));
+    }
+  } else if (sp.mixer == TL_MIXER_GDELTA) {
+    TL_REQUIRE(sp.decay_rank > 0 && sp.vdim == sp.dim && sp.kv_heads == sp.heads && sp.dim <= 256,
+               "tl_stack_create: layer %d: generalized delta rule with inner size %d, head sizes %d / %d (equal, at most 256), "
+               "%d key heads", i, sp.decay_rank, sp.dim, sp.vdim, sp.kv_heads);
+    TL_REQUIRE(sp.weights_of == 0 && own, "tl_stack_create: layer %d: a generalized delta layer owns its tensors", i);
+    const int hd = sp.heads * sp.dim;
+    L.qd = L.kd = L.vd = L.od = hd;
+    L.pd = 5 * hd + sp.decay_rank;
+    st->max_gd = hd > st->max_gd ? hd : st->max_gd;
+    ++st->gdelta_layers;
+    st->cache_bytes += sizeof(float) * (size_t)sp.heads * sp.dim * sp.dim;
+    L.expect.insert({"mix.r", "mix.k", "mix.v", "mix.g", "mix.a", "mix.a.b", "mix.w1", "mix.w2", "mix.w0", "mix.norm", "mix.o"});
+    TL_TRY(dev_alloc(st, &L.wa2, (size_t)hd * sp.decay_rank));
+    TL_TRY(dev_alloc(st, &L.w0, hd));
+    TL_TRY(dev_alloc(st, &L.a_bias, hd));
+    TL_TRY(dev_alloc(st, &L.onorm, hd));
+  } else if (sp.mixer == TL_MIXER_LINEAR) {
+    TL_REQUIRE(sp.kv_heads == sp.heads && sp.dim <= 256 && sp.vdim <= 512,
+               "tl_stack_create: layer %d: gated linear attention with %d / %d heads, sizes %d (at most 256) / %d (at most 512)", i,
+               sp.heads, sp.kv_heads, sp.dim, sp.vdim);
+    const int hd = sp.heads * sp.dim;
+    L.qd = L.kd = hd;  // q | forget gate
+    L.vd = L.od = sp.heads * sp.vdim;
+    L.pd = 2 * hd + L.vd;
+    st->max_dc = 2 * hd > st->max_dc ? 2 * hd : st->max_dc;
+    st->max_da = hd > st->max_da ? hd : st->max_da;
+    st->cache_bytes += sizeof(float) * (size_t)sp.heads * sp.vdim * sp.dim;
+    if (own) {
+      L.expect.insert({"mix.q", "mix.f", "mix.f.b", "mix.lower", "mix.v", "mix.norm", "mix.o"});
+      TL_TRY(dev_alloc(st, &L.lower, hd));
+      TL_TRY(dev_alloc(st, &L.f_bias, hd));
+      TL_TRY(dev_alloc(st, &L.onorm, sp.vdim));
+    }
+  } else {
+    const bool ph = sp.decay_per_head != 0;
+    TL_REQUIRE(sp.conv_taps >= 1 && sp.conv_taps <= 64 && (ph ? (sp.decay_rank == 0 && sp.gate_rank == 0) : (sp.decay_rank > 0 && sp.gate_rank > 0)),
+               "tl_stack_create: layer %d: %d taps, inner sizes %d / %d (none with a decay per head)", i, sp.conv_taps,
+               sp.decay_rank, sp.gate_rank);
+    TL_REQUIRE(sp.dim <= 256 && sp.vdim <= 512, "tl_stack_create: layer %d: key size %d above 256 or value size %d above 512", i,
+               sp.dim, sp.vdim);
+    L.qd = sp.kv_heads * sp.dim;  // queries share the keys' heads
+    L.kd = sp.kv_heads * sp.dim;
+    L.vd = sp.heads * sp.vdim;
+    L.od = sp.heads * sp.vdim;
+    // q | k | v | beta, then (a1 | g1) for the two-step projections or (a | gate) when they are direct
+    L.pd = L.qd + L.kd + L.vd + sp.heads + (ph ? sp.heads + L.vd : sp.decay_rank + sp.gate_rank);
+    L.gate_off = L.qd + L.kd + L.vd + 2 * sp.heads;
+    const int dc = L.qd + L.kd + L.vd, da = sp.heads * sp.dim;
+    st->max_dc = dc > st->max_dc ? dc : st->max_dc;
+    st->max_da = da > st->max_da ? da : st->max_da;
+    st->cache_bytes += sizeof(float) * ((size_t)sp.heads * sp.vdim * sp.dim + (size_t)(sp.conv_taps - 1) * dc);
+    if (own) {
+      L.expect.insert({"mix.q", "mix.k", "mix.v", "mix.b", "mix.o", "mix.q.conv", "mix.k.conv", "mix.v.conv", "mix.A_log",
+                       "mix.dt_bias", "mix.norm"});
+      if (ph) {
+        L.expect.insert({"mix.a", "mix.g"});
+      } else {
+        L.expect.insert({"mix.a1", "mix.g1", "mix.a2", "mix.g2"});
+        TL_TRY(dev_alloc(st, &L.wa2, (size_t)da * sp.decay_rank));
+        TL_TRY(dev_alloc(st, &L.wg2, (size_t)L.vd * sp.gate_rank));
+      }
+      TL_TRY(dev_alloc(st, &L.conv, (size_t)dc * sp.conv_taps));
+      TL_TRY(dev_alloc(st, &L.a_log, sp.heads));
+      TL_TRY(dev_alloc(st, &L.dt_bias, ph ? sp.heads : da));
+      TL_TRY(dev_alloc(st, &L.onorm, sp.vdim));
+    }
+  }
+  if (own) {
+    TL_TRY(dev_alloc(st, &L.wqkv, (size_t)L.pd * W));
+    TL_TRY(dev_alloc(st, &L.wo, W * L.od));
+  }
+  st->max_qkv = L.pd > st->max_qkv ? L.pd : st->max_qkv;
+  st->max_od = L.od > st->max_od ? L.od : st->max_od;
+  st->max_vd = L.vd > st->max_vd ? L.vd : st->max_vd;
+  st->max_heads = sp.heads > st->max_heads ? sp.heads : st->max_heads;
+  return 0;
+}
+
+// everything of layer i: block and feed-forward checks, the mixer (and the second mixer of a pair), norms, feed-forward tensors
+int setup_layer(TlStack* st, int i, int* first_mix) {
+  const tl_stack_config* cfg = &st->cfg;
+  Layer& L = st->layers[i];
+  const tl_layer_spec& sp = L.sp;
+  const size_t W = cfg->width;
+  const bool dyt = cfg->norm == TL_NORM_DYT, lnorm = cfg->norm == TL_NORM_LAYER, rms = cfg->norm == TL_NORM_RMS;
+  TL_REQUIRE((sp.block == TL_BLOCK_POST_NORM && !dyt && !lnorm && !rms) || (sp.block == TL_BLOCK_PARALLEL && dyt) ||
+                 (sp.block == TL_BLOCK_PRE_NORM && (lnorm || rms)),
+             "tl_stack_create: layer %d: block kind %d with norm kind %d (post-norm blocks take the one-plus RMS norm, parallel "
+             "blocks the Dynamic Tanh norm, pre-norm blocks the layer norm or the plain RMS norm)", i, sp.block, cfg->norm);
+  TL_REQUIRE(sp.mlp >= TL_MLP_NONE && sp.mlp <= TL_MLP_UNIT, "tl_stack_create: layer %d has feed-forward kind %d", i, sp.mlp);
+  TL_REQUIRE(sp.mlp != TL_MLP_DENSE || sp.block != TL_BLOCK_POST_NORM, "tl_stack_create: layer %d: a dense feed-forward "
+             "runs in parallel and pre-norm blocks only", i);
+  TL_REQUIRE(sp.mlp != TL_MLP_UNIT || sp.block == TL_BLOCK_PRE_NORM,
+             "tl_stack_create: layer %d: the plain up / activation / down unit runs in pre-norm blocks only", i);
+  TL_REQUIRE((sp.mixer != TL_MIXER_LATENT && sp.mixer != TL_MIXER_GDELTA && sp.mixer != TL_MIXER_LINEAR) || sp.block == TL_BLOCK_PRE_NORM,
+             "tl_stack_create: layer %d: latent attention, the generalized delta rule and gated linear attention run in "
+             "pre-norm blocks only", i);
+  TL_REQUIRE(sp.mixer != TL_MIXER_DELTA || sp.block != TL_BLOCK_POST_NORM, "tl_stack_create: layer %d: the delta rule runs "
+             "in parallel and pre-norm blocks only", i);
+  TL_REQUIRE(sp.glu == TL_GLU_SWISH || sp.glu == TL_GLU_RELU, "tl_stack_create: layer %d: gated unit of kind %d", i, sp.glu);
+  TL_REQUIRE(!L.side || sp.block == TL_BLOCK_PRE_NORM, "tl_stack_create: layer %d: two mixers side by side run in pre-norm blocks only", i);
+  L.wsrc = i;
+  if (sp.weights_of > 0) {
+    TL_REQUIRE(sp.weights_of - 1 < i, "tl_stack_create: layer %d takes its tensors from layer %d, which is not an earlier "
+               "layer", i, sp.weights_of - 1);
+    L.wsrc = st->layers[sp.weights_of - 1].wsrc;  // (a layer that itself borrows hands on the owner)
+    const Layer& O = st->layers[L.wsrc];
+    tl_layer_spec a = sp, b = O.sp;
+    a.weights_of = b.weights_of = 0;
+    a.side = b.side = nullptr;
+    bool same = memcmp(&a, &b, sizeof(a)) == 0 && !L.side == !O.side;
+    if (same && L.side) same = memcmp(&L.side->sp, &O.side->sp, sizeof(a)) == 0;
+    TL_REQUIRE(same, "tl_stack_create: layer %d differs from layer %d whose tensors it uses", i, L.wsrc);
+  }
+  const bool own = L.wsrc == i;
+  TL_TRY(setup_mixer(st, L, i, own, first_mix));
+  if (L.side) {
+    TL_REQUIRE(L.side->sp.mixer == TL_MIXER_SWA || L.side->sp.mixer == TL_MIXER_DELTA || L.side->sp.mixer == TL_MIXER_LINEAR,
+               "tl_stack_create: layer %d: a second mixer of kind %d", i, L.side->sp.mixer);
+    TL_REQUIRE(!L.side->sp.v_mix && !sp.v_mix, "tl_stack_create: layer %d: value mixing inside a pair of mixers", i);
+    L.side->wsrc = L.wsrc;
+    TL_TRY(setup_mixer(st, *L.side, i, own, first_mix));
+    st->any_pair = true;
+  }
+  if (own) {
+    TL_TRY(dev_alloc(st, &L.norm1, W));
+    TL_TRY(dev_alloc(st, &L.norm2, W));
+    L.expect.insert("norm1");
+    if (lnorm) {
+      TL_TRY(dev_alloc(st, &L.norm1_b, W));
+      TL_TRY(dev_alloc(st, &L.norm2_b, W));
+      L.expect.insert("norm1.b");
+    }
+    if (dyt) {
+      TL_TRY(dev_alloc(st, &L.norm1_b, W));
+      TL_TRY(dev_alloc(st, &L.norm1_alpha, 1));
+      L.expect.insert({"norm1.b", "norm1.alpha"});
+    }
+    if (cfg->canon_taps > 0) {
+      TL_TRY(dev_alloc(st, &L.canon1, W * cfg->canon_taps));
+      L.expect.insert("canon1");
+      if (sp.mlp != TL_MLP_NONE) {
+        TL_TRY(dev_alloc(st, &L.canon2, W * cfg->canon_taps));
+        L.expect.insert("canon2");
+      } else {
+        L.optional.insert("canon2");
+      }
+    }
+  }
+  if (cfg->canon_taps > 1) st->cache_bytes += sizeof(float) * (size_t)(cfg->canon_taps - 1) * W * (sp.mlp != TL_MLP_NONE ? 2 : 1);
+  // ---- feed-forward ----
+  const bool pre_rms = sp.block == TL_BLOCK_PRE_NORM && rms;
+  if (sp.mlp == TL_MLP_MOE) {
+    TL_REQUIRE(sp.block != TL_BLOCK_PRE_NORM || rms, "tl_stack_create: layer %d: routed experts behind a layer norm", i);
+    TL_REQUIRE(sp.experts > 0 && sp.top > 0 && sp.top <= sp.experts && sp.expert_ff > 0 && sp.shared_ff >= 0,
+               "tl_stack_create: layer %d: %d experts, top %d, sizes %d / %d", i, sp.experts, sp.top, sp.expert_ff, sp.shared_ff);
+    TL_REQUIRE(sp.route == TL_ROUTE_TOP_LOGITS ||
+                   ((sp.route == TL_ROUTE_SOFTMAX_GROUPS || sp.route == TL_ROUTE_SIGMOID_GROUPS) && sp.route_groups > 0 &&
+                    sp.experts % sp.route_groups == 0 && sp.route_keep > 0 && sp.route_keep <= sp.route_groups &&
+                    (long long)sp.route_keep * (sp.experts / sp.route_groups) >= sp.top),
+               "tl_stack_create: layer %d: router kind %d, %d experts in %d groups, %d kept, top %d", i, sp.route, sp.experts,
+               sp.route_groups, sp.route_keep, sp.top);
+    TL_REQUIRE(!sp.shared_gate || sp.shared_ff > 0, "tl_stack_create: layer %d: a gate without a shared expert", i);
+    TL_REQUIRE(!pre_rms || !sp.shared_gate, "tl_stack_create: layer %d: a gated shared expert runs in parallel blocks only", i);
+    if (own) {
+      if (sp.block == TL_BLOCK_POST_NORM || pre_rms) L.expect.insert("norm2");
+      L.expect.insert("mlp.router");
+      if (sp.route == TL_ROUTE_TOP_LOGITS) L.expect.insert("mlp.router.b");
+      if (sp.route == TL_ROUTE_SIGMOID_GROUPS) L.expect.insert("mlp.correction");
+      for (int e = 0; e < sp.experts; ++e)
+        for (const char* k : {"gate", "up", "down"}) L.expect.insert("mlp.e" + std::to_string(e) + "." + k);
+      TL_TRY(dev_alloc(st, &L.router, (size_t)sp.experts * W));
+      TL_TRY(dev_alloc(st, &L.router_b, sp.experts));
+      TL_TRY(dev_alloc(st, &L.gu, (size_t)sp.experts * 2 * sp.expert_ff * W));
+      TL_TRY(dev_alloc(st, &L.down, (size_t)sp.experts * W * sp.expert_ff));
+      if (sp.shared_ff) {
+        L.expect.insert({"mlp.shared.gate", "mlp.shared.up", "mlp.shared.down"});
+        TL_TRY(dev_alloc(st, &L.sgu, (size_t)2 * sp.shared_ff * W));
+        TL_TRY(dev_alloc(st, &L.sdown, W * sp.shared_ff));
+        if (sp.shared_gate) {
+          L.expect.insert("mlp.shared.sg");
+          TL_TRY(dev_alloc(st, &L.sg, W));
+        }
+      }
+    }
+    st->max_top = sp.top > st->max_top ? sp.top : st->max_top;
+    st->max_experts = sp.experts > st->max_experts ? sp.experts : st->max_experts;
+    st->max_gu = 2 * sp.expert_ff * sp.top > st->max_gu ? 2 * sp.expert_ff * sp.top : st->max_gu;
+    st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
+  } else if (sp.mlp == TL_MLP_DENSE) {
+    TL_REQUIRE(sp.block != TL_BLOCK_PRE_NORM || rms, "tl_stack_create: layer %d: a gated unit behind a layer norm", i);
+    TL_REQUIRE(sp.shared_ff > 0, "tl_stack_create: layer %d: a dense feed-forward of size %d", i, sp.shared_ff);
+    if (own) {
+      if (pre_rms) L.expect.insert("norm2");
+      L.expect.insert({"mlp.gate", "mlp.up", "mlp.down"});
+      TL_TRY(dev_alloc(st, &L.sgu, (size_t)2 * sp.shared_ff * W));
+      TL_TRY(dev_alloc(st, &L.sdown, W * sp.shared_ff));
+    }
+    st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
+  } else if (sp.mlp == TL_MLP_UNIT) {
+    TL_REQUIRE(lnorm, "tl_stack_create: layer %d: the plain up / activation / down unit sits behind a layer norm", i);
+    TL_REQUIRE(sp.shared_ff > 0 && sp.act >= TL_ACT_NONE && sp.act <= TL_ACT_TANH,
+               "tl_stack_create: layer %d: a feed-forward of size %d with activation kind %d", i, sp.shared_ff, sp.act);
+    if (own) {
+      L.expect.insert({"norm2", "norm2.b", "mlp.up", "mlp.down"});
+      if (sp.act == TL_ACT_XIELU) L.expect.insert("mlp.act");
+      TL_TRY(dev_alloc(st, &L.sgu, (size_t)sp.shared_ff * W));
+      TL_TRY(dev_alloc(st, &L.sdown, W * sp.shared_ff));
+    }
+    st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
+  } else if (own) {
+    L.optional.insert("norm2");
+    if (lnorm) L.optional.insert("norm2.b");
+  }
+  return 0;
+}
+
+}  // namespace
+
 int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
   TL_REQUIRE(cfg && out && cfg->layers, "tl_stack_create: null argument");
   TL_REQUIRE(cfg->width > 0 && cfg->vocab > 0 && cfg->n_layers > 0 && cfg->max_positions > 0,
              "tl_stack_create: non-positive size in the configuration");
-  TL_REQUIRE(cfg->norm == TL_NORM_RMS_ONE_PLUS || cfg->norm == TL_NORM_DYT || cfg->norm == TL_NORM_LAYER,
-             "tl_stack_create: norm kind %d", cfg->norm);
+  TL_REQUIRE(cfg->norm >= TL_NORM_RMS_ONE_PLUS && cfg->norm <= TL_NORM_RMS, "tl_stack_create: norm kind %d", cfg->norm);
+  TL_REQUIRE(cfg->canon_taps >= 0 && cfg->canon_taps <= 64 && (cfg->canon_taps == 0 || cfg->norm == TL_NORM_RMS),
+             "tl_stack_create: %d taps on what the sublayers read (a convolution there follows the plain RMS norm)", cfg->canon_taps);
+  TL_REQUIRE(cfg->norm != TL_NORM_RMS || !cfg->embed_norm, "tl_stack_create: an embedding norm with the plain RMS norm");
   TlStack* st = new TlStack();
   st->cfg = *cfg;
   st->layers.resize(cfg->n_layers);
@@ -195,272 +572,17 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
     tl_stack_free(st);
     return code;
   };
-#define CREATE_REQUIRE(cond, ...) \
-  do {                            \
-    if (!(cond)) {                \
-      tl_set_error(__VA_ARGS__);  \
-      return fail(2);             \
-    }                             \
-  } while (0)
   for (int i = 0; i < cfg->n_layers && rc == 0; ++i) {
     Layer& L = st->layers[i];
     L.sp = cfg->layers[i];
-    const tl_layer_spec& sp = L.sp;
-    const bool dyt = cfg->norm == TL_NORM_DYT, lnorm = cfg->norm == TL_NORM_LAYER;
-    CREATE_REQUIRE(sp.mixer >= TL_MIXER_SWA && sp.mixer <= TL_MIXER_GDELTA,
-                   "tl_stack_create: layer %d has mixer kind %d; this engine has windowed attention (%d), the gated delta rule (%d), "
-                   "latent attention (%d) and the generalized delta rule (%d)",
-                   i, sp.mixer, TL_MIXER_SWA, TL_MIXER_DELTA, TL_MIXER_LATENT, TL_MIXER_GDELTA);
-    CREATE_REQUIRE(sp.heads > 0 && sp.kv_heads > 0 && sp.heads % sp.kv_heads == 0 && sp.dim > 0 && sp.vdim > 0,
-                   "tl_stack_create: layer %d: %d heads / %d key-value heads / sizes %d, %d", i, sp.heads, sp.kv_heads, sp.dim, sp.vdim);
-    CREATE_REQUIRE((sp.block == TL_BLOCK_POST_NORM && !dyt && !lnorm) || (sp.block == TL_BLOCK_PARALLEL && dyt) ||
-                       (sp.block == TL_BLOCK_PRE_NORM && lnorm),
-                   "tl_stack_create: layer %d: block kind %d with norm kind %d (post-norm blocks take the RMS norm, parallel "
-                   "blocks the Dynamic Tanh norm, pre-norm blocks the layer norm)", i, sp.block, cfg->norm);
-    CREATE_REQUIRE(sp.mlp >= TL_MLP_NONE && sp.mlp <= TL_MLP_UNIT, "tl_stack_create: layer %d has feed-forward kind %d", i, sp.mlp);
-    CREATE_REQUIRE(sp.mlp != TL_MLP_DENSE || sp.block == TL_BLOCK_PARALLEL, "tl_stack_create: layer %d: a dense feed-forward "
-                   "runs in parallel blocks only", i);
-    CREATE_REQUIRE(sp.mlp == TL_MLP_NONE || (sp.mlp == TL_MLP_UNIT) == (sp.block == TL_BLOCK_PRE_NORM),
-                   "tl_stack_create: layer %d: feed-forward kind %d in block kind %d (pre-norm blocks take the plain up / "
-                   "activation / down unit, and only they)", i, sp.mlp, sp.block);
-    CREATE_REQUIRE((sp.mixer != TL_MIXER_LATENT && sp.mixer != TL_MIXER_GDELTA) || sp.block == TL_BLOCK_PRE_NORM,
-                   "tl_stack_create: layer %d: latent attention and the generalized delta rule run in pre-norm blocks only", i);
-    CREATE_REQUIRE(sp.mixer != TL_MIXER_DELTA || sp.block == TL_BLOCK_PARALLEL, "tl_stack_create: layer %d: the delta rule runs "
-                   "in parallel blocks only", i);
-    L.wsrc = i;
-    if (sp.weights_of > 0) {
-      CREATE_REQUIRE(sp.weights_of - 1 < i, "tl_stack_create: layer %d takes its tensors from layer %d, which is not an earlier "
-                     "layer", i, sp.weights_of - 1);
-      L.wsrc = st->layers[sp.weights_of - 1].wsrc;  // (a layer that itself borrows hands on the owner)
-      tl_layer_spec a = sp, b = st->layers[L.wsrc].sp;
-      a.weights_of = b.weights_of = 0;
-      CREATE_REQUIRE(memcmp(&a, &b, sizeof(a)) == 0, "tl_stack_create: layer %d differs from layer %d whose tensors it uses", i, L.wsrc);
+    if (L.sp.side) {  // the second mixer's entry is copied: the caller's may not outlive this call
+      L.side.reset(new Layer());
+      L.side->sp = *L.sp.side;
+      L.side->sp.side = nullptr;
+      L.sp.side = &L.side->sp;
     }
-    const bool own = L.wsrc == i;
-    // ---- mixer ----
-    if (sp.mixer == TL_MIXER_SWA) {
-      CREATE_REQUIRE(!sp.values_are_keys || sp.vdim == sp.dim, "tl_stack_create: layer %d: values that are keys need vdim == dim", i);
-      CREATE_REQUIRE(sp.rot_dims >= 0 && sp.rot_dims <= sp.dim && (sp.rot_dims & 1) == 0 && (sp.rot_dims == 0 || sp.rot_base > 0.0f),
-                     "tl_stack_create: layer %d: %d rotating dimensions of %d, base %g", i, sp.rot_dims, sp.dim, sp.rot_base);
-      CREATE_REQUIRE(sp.keep_first >= 0, "tl_stack_create: layer %d: %d kept first keys", i, sp.keep_first);
-      CREATE_REQUIRE(sp.attn_weight >= TL_ATTN_SOFTMAX && sp.attn_weight <= TL_ATTN_SOFTMAX_SINK && sp.q_temp_every >= 0,
-                     "tl_stack_create: layer %d: attention weights of kind %d, query temperature every %d", i, sp.attn_weight,
-                     sp.q_temp_every);
-      L.rotary_path = sp.rot_dims > 0 || sp.qk_norm == TL_QK_NORM_HEAD_UNIT || sp.values_are_keys;
-      CREATE_REQUIRE(!L.rotary_path || (sp.qk_norm != TL_QK_NORM_WHOLE && !sp.v_mix && sp.q_temp_every == 0),
-                     "tl_stack_create: layer %d: rotation / per-head norm / values-are-keys do not combine with the "
-                     "whole-projection norm, value mixing or a query temperature", i);
-      CREATE_REQUIRE(sp.qk_norm >= TL_QK_NORM_NONE && sp.qk_norm <= TL_QK_NORM_HEAD_UNIT, "tl_stack_create: layer %d: q/k norm %d", i, sp.qk_norm);
-      L.qd = sp.heads * sp.dim;
-      L.kd = sp.kv_heads * sp.dim;
-      L.vd = sp.kv_heads * sp.vdim;
-      L.od = sp.heads * sp.vdim;
-      L.pd = L.qd + L.kd + (sp.values_are_keys ? 0 : L.vd);
-      if (sp.v_mix) {
-        if (first_mix < 0) {
-          first_mix = i;
-          L.vmix_mode = 1;
-        } else {
-          L.vmix_mode = 2;
-          CREATE_REQUIRE(st->layers[first_mix].vd == L.vd, "tl_stack_create: layer %d mixes %d values with the %d of layer %d", i,
-                         L.vd, st->layers[first_mix].vd, first_mix);
-        }
-      }
-      st->cache_bytes += sizeof(float) * (size_t)cfg->max_positions * (L.kd + L.vd);
-      if (own) {
-        L.expect.insert({"mix.q", "mix.k", "mix.o"});
-        if (!sp.values_are_keys) L.expect.insert("mix.v");
-        if (sp.qk_norm == TL_QK_NORM_WHOLE) L.expect.insert({"mix.q.norm", "mix.k.norm"});
-        else L.optional.insert({"mix.q.norm", "mix.k.norm"});
-        if (L.vmix_mode == 2) L.expect.insert("mix.vmix");
-        else L.optional.insert("mix.vmix");
-        if (sp.attn_weight == TL_ATTN_SIGMOID) L.expect.insert("mix.pb");
-        if ((rc = dev_alloc(st, &L.q_norm, L.qd))) break;
-        if ((rc = dev_alloc(st, &L.k_norm, L.kd))) break;
-        if ((rc = dev_alloc(st, &L.lambda, 1))) break;
-        if ((rc = dev_alloc(st, &L.pb, sp.heads))) break;
-        if (sp.rot_dims > 0) {
-          std::vector<double> f(sp.rot_dims / 2);
-          tl_rotary_frequencies(sp.rot_dims, sp.rot_base, sp.rot_factor, sp.rot_original, sp.rot_fast, sp.rot_slow, f.data(), &L.mscale);
-          if ((rc = dev_alloc(st, &L.freq, f.size()))) break;
-          if (hipMemcpy(L.freq, f.data(), sizeof(double) * f.size(), hipMemcpyHostToDevice) != hipSuccess) {
-            tl_set_error("tl_stack_create: upload of the rotary frequencies failed");
-            return fail(1);
-          }
-        }
-      }
-    } else if (sp.mixer == TL_MIXER_LATENT) {
-      CREATE_REQUIRE(sp.q_rank > 0 && sp.kv_rank > 0 && sp.rot_dim >= 0 && sp.rot_dims >= 0 && sp.rot_dims <= sp.rot_dim &&
-                         (sp.rot_dims & 1) == 0 && (sp.rot_dims == 0 || sp.rot_base > 0.0f) && sp.kv_heads == sp.heads,
-                     "tl_stack_create: layer %d: latents of %d / %d, %d rotated dimensions of which %d turn (base %g), %d key heads",
-                     i, sp.q_rank, sp.kv_rank, sp.rot_dim, sp.rot_dims, sp.rot_base, sp.kv_heads);
-      CREATE_REQUIRE(sp.kv_rank <= 512, "tl_stack_create: layer %d: a key/value latent of %d above 512", i, sp.kv_rank);
-      CREATE_REQUIRE(sp.weights_of == 0, "tl_stack_create: layer %d: a latent layer owns its tensors (it may share a cache: kv_from)", i);
-      L.kv_src = i;
-      if (sp.kv_from > 0) {
-        const int j = sp.kv_from - 1;
-        CREATE_REQUIRE(j < i && st->layers[j].sp.mixer == TL_MIXER_LATENT && st->layers[j].sp.kv_from == 0,
-                       "tl_stack_create: layer %d reads the latent cache of layer %d, which is not an earlier latent layer "
-                       "with a projection of its own", i, j);
-        const tl_layer_spec& o = st->layers[j].sp;
-        CREATE_REQUIRE(o.kv_rank == sp.kv_rank && o.rot_dim == sp.rot_dim && o.rot_dims == sp.rot_dims && o.rot_base == sp.rot_base,
-                       "tl_stack_create: layer %d and layer %d, whose latent cache it reads, differ in latent size or rotation", i, j);
-        L.kv_src = j;
-      }
-      const bool own_kv = L.kv_src == i;
-      const int qh = sp.dim + sp.rot_dim, ah = sp.kv_rank + sp.rot_dim;
-      L.qd = sp.heads * qh;
-      L.kd = own_kv ? sp.kv_rank + sp.rot_dim : 0;
-      L.vd = 0;
-      L.od = sp.heads * sp.vdim;
-      L.gate_off = sp.q_rank + L.kd;
-      L.pd = L.gate_off + (sp.head_gate ? sp.heads : 0);
-      if (own_kv) st->cache_bytes += sizeof(float) * (size_t)cfg->max_positions * L.kd;
-      st->max_lq = L.qd > st->max_lq ? L.qd : st->max_lq;
-      st->max_lqa = sp.heads * ah > st->max_lqa ? sp.heads * ah : st->max_lqa;
-      st->max_lk = sp.heads * qh > st->max_lk ? sp.heads * qh : st->max_lk;
-      st->max_lv = sp.heads * sp.vdim > st->max_lv ? sp.heads * sp.vdim : st->max_lv;
-      st->max_od = sp.heads * sp.kv_rank > st->max_od ? sp.heads * sp.kv_rank : st->max_od;  // the weighted latents of all heads
-      L.expect.insert({"mix.dq", "mix.dq.norm", "mix.uq", "mix.uk", "mix.uv", "mix.o"});
-      if (own_kv) L.expect.insert({"mix.dkv", "mix.dkv.norm"});
-      if (sp.head_gate) L.expect.insert("mix.g");
-      if ((rc = dev_alloc(st, &L.wuq, (size_t)L.qd * sp.q_rank))) break;
-      if ((rc = dev_alloc(st, &L.wukt, (size_t)sp.heads * sp.kv_rank * sp.dim))) break;
-      if ((rc = dev_alloc(st, &L.wuk, (size_t)sp.heads * sp.kv_rank * sp.dim))) break;
-      if ((rc = dev_alloc(st, &L.wuv, (size_t)sp.heads * sp.vdim * sp.kv_rank))) break;
-      if ((rc = dev_alloc(st, &L.dq_norm, sp.q_rank))) break;
-      if ((rc = dev_alloc(st, &L.dkv_norm, sp.kv_rank))) break;
-      if (sp.rot_dims > 0) {
-        std::vector<double> f(sp.rot_dims / 2);
-        float unused = 1.0f;
-        tl_rotary_frequencies(sp.rot_dims, sp.rot_base, 0.0, 0.0, 0.0, 0.0, f.data(), &unused);
-        if ((rc = dev_alloc(st, &L.freq, f.size()))) break;
-        if (hipMemcpy(L.freq, f.data(), sizeof(double) * f.size(), hipMemcpyHostToDevice) != hipSuccess) {
-          tl_set_error("tl_stack_create: upload of the rotary frequencies failed");
-          return fail(1);
-        }
-      }
-    } else if (sp.mixer == TL_MIXER_GDELTA) {
-      CREATE_REQUIRE(sp.decay_rank > 0 && sp.vdim == sp.dim && sp.kv_heads == sp.heads && sp.dim <= 256,
-                     "tl_stack_create: layer %d: generalized delta rule with inner size %d, head sizes %d / %d (equal, at most 256), "
-                     "%d key heads", i, sp.decay_rank, sp.dim, sp.vdim, sp.kv_heads);
-      CREATE_REQUIRE(sp.weights_of == 0, "tl_stack_create: layer %d: a generalized delta layer owns its tensors", i);
-      const int hd = sp.heads * sp.dim;
-      L.qd = L.kd = L.vd = L.od = hd;
-      L.pd = 5 * hd + sp.decay_rank;
-      st->max_gd = hd > st->max_gd ? hd : st->max_gd;
-      ++st->gdelta_layers;
-      st->cache_bytes += sizeof(float) * (size_t)sp.heads * sp.dim * sp.dim;
-      L.expect.insert({"mix.r", "mix.k", "mix.v", "mix.g", "mix.a", "mix.a.b", "mix.w1", "mix.w2", "mix.w0", "mix.norm", "mix.o"});
-      if ((rc = dev_alloc(st, &L.wa2, (size_t)hd * sp.decay_rank))) break;
-      if ((rc = dev_alloc(st, &L.w0, hd))) break;
-      if ((rc = dev_alloc(st, &L.a_bias, hd))) break;
-      if ((rc = dev_alloc(st, &L.onorm, hd))) break;
-    } else {
-      CREATE_REQUIRE(sp.conv_taps >= 1 && sp.conv_taps <= 64 && sp.decay_rank > 0 && sp.gate_rank > 0,
-                     "tl_stack_create: layer %d: %d taps, inner sizes %d / %d", i, sp.conv_taps, sp.decay_rank, sp.gate_rank);
-      CREATE_REQUIRE(sp.dim <= 256 && sp.vdim <= 512, "tl_stack_create: layer %d: key size %d above 256 or value size %d above 512", i,
-                     sp.dim, sp.vdim);
-      L.qd = sp.kv_heads * sp.dim;  // queries share the keys' heads
-      L.kd = sp.kv_heads * sp.dim;
-      L.vd = sp.heads * sp.vdim;
-      L.od = sp.heads * sp.vdim;
-      L.pd = L.qd + L.kd + L.vd + sp.heads + sp.decay_rank + sp.gate_rank;
-      const int dc = L.qd + L.kd + L.vd, da = sp.heads * sp.dim;
-      st->max_dc = dc > st->max_dc ? dc : st->max_dc;
-      st->max_da = da > st->max_da ? da : st->max_da;
-      st->cache_bytes += sizeof(float) * ((size_t)sp.heads * sp.vdim * sp.dim + (size_t)(sp.conv_taps - 1) * dc);
-      if (own) {
-        L.expect.insert({"mix.q", "mix.k", "mix.v", "mix.b", "mix.a1", "mix.g1", "mix.a2", "mix.g2", "mix.o", "mix.q.conv",
-                         "mix.k.conv", "mix.v.conv", "mix.A_log", "mix.dt_bias", "mix.norm"});
-        if ((rc = dev_alloc(st, &L.wa2, (size_t)da * sp.decay_rank))) break;
-        if ((rc = dev_alloc(st, &L.wg2, (size_t)L.vd * sp.gate_rank))) break;
-        if ((rc = dev_alloc(st, &L.conv, (size_t)dc * sp.conv_taps))) break;
-        if ((rc = dev_alloc(st, &L.a_log, sp.heads))) break;
-        if ((rc = dev_alloc(st, &L.dt_bias, da))) break;
-        if ((rc = dev_alloc(st, &L.onorm, sp.vdim))) break;
-      }
-    }
-    if (own) {
-      if ((rc = dev_alloc(st, &L.wqkv, (size_t)L.pd * W))) break;
-      if ((rc = dev_alloc(st, &L.wo, W * L.od))) break;
-      if ((rc = dev_alloc(st, &L.norm1, W))) break;
-      if ((rc = dev_alloc(st, &L.norm2, W))) break;
-      L.expect.insert("norm1");
-      if (lnorm) {
-        if ((rc = dev_alloc(st, &L.norm1_b, W))) break;
-        if ((rc = dev_alloc(st, &L.norm2_b, W))) break;
-        L.expect.insert("norm1.b");
-      }
-      if (dyt) {
-        if ((rc = dev_alloc(st, &L.norm1_b, W))) break;
-        if ((rc = dev_alloc(st, &L.norm1_alpha, 1))) break;
-        L.expect.insert({"norm1.b", "norm1.alpha"});
-      }
-    }
-    // ---- feed-forward ----
-    if (sp.mlp == TL_MLP_MOE) {
-      CREATE_REQUIRE(sp.experts > 0 && sp.top > 0 && sp.top <= sp.experts && sp.expert_ff > 0 && sp.shared_ff >= 0,
-                     "tl_stack_create: layer %d: %d experts, top %d, sizes %d / %d", i, sp.experts, sp.top, sp.expert_ff, sp.shared_ff);
-      CREATE_REQUIRE(sp.route == TL_ROUTE_TOP_LOGITS ||
-                         (sp.route == TL_ROUTE_SOFTMAX_GROUPS && sp.route_groups > 0 && sp.experts % sp.route_groups == 0 &&
-                          sp.route_keep > 0 && sp.route_keep <= sp.route_groups &&
-                          (long long)sp.route_keep * (sp.experts / sp.route_groups) >= sp.top),
-                     "tl_stack_create: layer %d: router kind %d, %d experts in %d groups, %d kept, top %d", i, sp.route, sp.experts,
-                     sp.route_groups, sp.route_keep, sp.top);
-      CREATE_REQUIRE(!sp.shared_gate || sp.shared_ff > 0, "tl_stack_create: layer %d: a gate without a shared expert", i);
-      if (own) {
-        if (sp.block == TL_BLOCK_POST_NORM) L.expect.insert("norm2");
-        L.expect.insert("mlp.router");
-        if (sp.route == TL_ROUTE_TOP_LOGITS) L.expect.insert("mlp.router.b");
-        for (int e = 0; e < sp.experts; ++e)
-          for (const char* k : {"gate", "up", "down"}) L.expect.insert("mlp.e" + std::to_string(e) + "." + k);
-        if ((rc = dev_alloc(st, &L.router, (size_t)sp.experts * W))) break;
-        if ((rc = dev_alloc(st, &L.router_b, sp.experts))) break;
-        if ((rc = dev_alloc(st, &L.gu, (size_t)sp.experts * 2 * sp.expert_ff * W))) break;
-        if ((rc = dev_alloc(st, &L.down, (size_t)sp.experts * W * sp.expert_ff))) break;
-        if (sp.shared_ff) {
-          L.expect.insert({"mlp.shared.gate", "mlp.shared.up", "mlp.shared.down"});
-          if ((rc = dev_alloc(st, &L.sgu, (size_t)2 * sp.shared_ff * W))) break;
-          if ((rc = dev_alloc(st, &L.sdown, W * sp.shared_ff))) break;
-          if (sp.shared_gate) {
-            L.expect.insert("mlp.shared.sg");
-            if ((rc = dev_alloc(st, &L.sg, W))) break;
-          }
-        }
-      }
-      st->max_top = sp.top > st->max_top ? sp.top : st->max_top;
-      st->max_experts = sp.experts > st->max_experts ? sp.experts : st->max_experts;
-      st->max_gu = 2 * sp.expert_ff * sp.top > st->max_gu ? 2 * sp.expert_ff * sp.top : st->max_gu;
-      st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
-    } else if (sp.mlp == TL_MLP_DENSE) {
-      CREATE_REQUIRE(sp.shared_ff > 0, "tl_stack_create: layer %d: a dense feed-forward of size %d", i, sp.shared_ff);
-      if (own) {
-        L.expect.insert({"mlp.gate", "mlp.up", "mlp.down"});
-        if ((rc = dev_alloc(st, &L.sgu, (size_t)2 * sp.shared_ff * W))) break;
-        if ((rc = dev_alloc(st, &L.sdown, W * sp.shared_ff))) break;
-      }
-      st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
-    } else if (sp.mlp == TL_MLP_UNIT) {
-      CREATE_REQUIRE(sp.shared_ff > 0 && sp.act >= TL_ACT_NONE && sp.act <= TL_ACT_TANH,
-                     "tl_stack_create: layer %d: a feed-forward of size %d with activation kind %d", i, sp.shared_ff, sp.act);
-      if (own) {
-        L.expect.insert({"norm2", "norm2.b", "mlp.up", "mlp.down"});
-        if (sp.act == TL_ACT_XIELU) L.expect.insert("mlp.act");
-        if ((rc = dev_alloc(st, &L.sgu, (size_t)sp.shared_ff * W))) break;
-        if ((rc = dev_alloc(st, &L.sdown, W * sp.shared_ff))) break;
-      }
-      st->max_sff = sp.shared_ff > st->max_sff ? sp.shared_ff : st->max_sff;
-    } else if (own) {
-      L.optional.insert("norm2");
-      if (lnorm) L.optional.insert("norm2.b");
-    }
-    st->max_qkv = L.pd > st->max_qkv ? L.pd : st->max_qkv;
-    st->max_od = L.od > st->max_od ? L.od : st->max_od;
-    st->max_vd = L.vd > st->max_vd ? L.vd : st->max_vd;
-    st->max_heads = sp.heads > st->max_heads ? sp.heads : st->max_heads;
+    rc = setup_layer(st, i, &first_mix);
   }
-#undef CREATE_REQUIRE
   if (rc) return fail(rc);
   if ((rc = dev_alloc(st, &st->embed, (size_t)cfg->vocab * W)) || (rc = dev_alloc(st, &st->head, (size_t)cfg->vocab * W)) ||
       (rc = dev_alloc(st, &st->embed_norm, W)) || (rc = dev_alloc(st, &st->final_norm, W)) ||
@@ -527,9 +649,20 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
   int li = -1, used = 0;
   TL_REQUIRE(sscanf(name, "l%d.%n", &li, &used) == 1 && used > 0 && li >= 0 && li < st->cfg.n_layers,
              "tl_stack_set_tensor: no place for a tensor named %s", name);
-  Layer& L = st->layers[li];
+  Layer* target = &st->layers[li];
+  std::string r = n.substr(used);
+  if (target->side) {  // two mixers side by side: mix.left.* is the first mixer's mix.*, mix.right.* the second's
+    if (r.compare(0, 9, "mix.left.") == 0) {
+      r = "mix." + r.substr(9);
+    } else if (r.compare(0, 10, "mix.right.") == 0) {
+      r = "mix." + r.substr(10);
+      target = target->side.get();
+    } else {
+      TL_REQUIRE(r.compare(0, 4, "mix.") != 0, "tl_stack_set_tensor: %s: the mixers of layer %d are mix.left and mix.right", name, li);
+    }
+  }
+  Layer& L = *target;
   const tl_layer_spec& sp = L.sp;
-  const std::string r = n.substr(used);
   if (L.optional.count(r) && !L.expect.count(r)) {  // present in the checkpoint, not used by this configuration: checked, dropped
     return 0;
   }
@@ -540,6 +673,58 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
   if (r == "norm1.alpha") VECTOR(L.norm1_alpha, 1);
   if (r == "norm2") VECTOR(L.norm2, W);
   if (r == "norm2.b") VECTOR(L.norm2_b, W);
+  if (r == "canon1") MATRIX(L.canon1, W, st->cfg.canon_taps);
+  if (r == "canon2") MATRIX(L.canon2, W, st->cfg.canon_taps);
+  if (sp.mixer == TL_MIXER_LINEAR) {
+    const long long hd = (long long)sp.heads * sp.dim;
+    if (r == "mix.q") MATRIX(L.wqkv, hd, W);
+    if (r == "mix.f") MATRIX(L.wqkv + (size_t)hd * W, hd, W);
+    if (r == "mix.v") MATRIX(L.wqkv + (size_t)2 * hd * W, L.vd, W);
+    if (r == "mix.f.b") VECTOR(L.f_bias, hd);
+    if (r == "mix.lower") VECTOR(L.lower, hd);
+    if (r == "mix.norm") VECTOR(L.onorm, sp.vdim);
+    if (r == "mix.o") MATRIX(L.wo, W, L.od);
+  }
+  if (sp.mixer == TL_MIXER_SWA) {
+    const long long hd = sp.dim, taps = sp.qkv_conv;
+    if (sp.qk_norm == TL_QK_NORM_HEAD_RMS) {
+      if (r == "mix.q.norm") VECTOR(L.q_norm, hd);
+      if (r == "mix.k.norm") VECTOR(L.k_norm, hd);
+    }
+    if (r == "mix.g") MATRIX(L.wqkv + (size_t)L.gate_off * W, L.od, W);
+    if (r == "mix.q.b") VECTOR(L.qkv_b, L.qd);
+    if (r == "mix.k.b") VECTOR(L.qkv_b + L.qd, L.kd);
+    if (r == "mix.v.b") VECTOR(L.qkv_b + L.qd + L.kd, L.vd);
+    if (r == "mix.q.conv") MATRIX(L.conv, L.qd, taps);
+    if (r == "mix.k.conv") MATRIX(L.conv + (size_t)L.qd * taps, L.kd, taps);
+    if (r == "mix.v.conv") MATRIX(L.conv + (size_t)(L.qd + L.kd) * taps, L.vd, taps);
+    if (r == "mix.r1") VECTOR(L.r1, sp.heads);
+    if (r == "mix.r2") VECTOR(L.r2, sp.heads);
+    if (r == "mix.sink") VECTOR(L.sinkv, sp.heads);
+    for (int j = 0; j < 4; ++j) {
+      static const char* const names[4] = {"mix.lq1", "mix.lk1", "mix.lq2", "mix.lk2"};
+      if (r != names[j]) continue;
+      TL_REQUIRE(shape_is(shape, ndim, hd), "tl_stack_set_tensor: %s does not have %lld elements", name, hd);
+      L.lvec[j].resize((size_t)hd);
+      for (long long d = 0; d < hd; ++d) {
+        if (type == TL_BF16) {
+          const uint32_t bits = (uint32_t) static_cast<const uint16_t*>(host)[d] << 16;
+          memcpy(&L.lvec[j][d], &bits, 4);
+        } else {
+          L.lvec[j][d] = static_cast<const float*>(host)[d];
+        }
+      }
+      if (L.expect.count("mix.lq1") + L.expect.count("mix.lk1") + L.expect.count("mix.lq2") + L.expect.count("mix.lk2") == 0) {
+        double d1 = 0.0, d2 = 0.0;  // lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff_init: one number for the layer, formed once
+        for (long long d = 0; d < hd; ++d) {
+          d1 += (double)L.lvec[0][d] * L.lvec[1][d];
+          d2 += (double)L.lvec[2][d] * L.lvec[3][d];
+        }
+        L.lam = (float)(exp(d1) - exp(d2) + (double)sp.diff_init);
+      }
+      return 0;
+    }
+  }
   if (sp.mixer == TL_MIXER_LATENT) {
     const long long qh = sp.dim + sp.rot_dim;
     if (r == "mix.dq") MATRIX(L.wqkv, sp.q_rank, W);
@@ -609,6 +794,11 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
   if (sp.mixer == TL_MIXER_DELTA) {
     const long long c0 = L.qd + L.kd + L.vd, da = (long long)sp.heads * sp.dim, taps = sp.conv_taps;
     if (r == "mix.b") MATRIX(L.wqkv + (size_t)c0 * W, sp.heads, W);
+    if (sp.decay_per_head) {
+      if (r == "mix.a") MATRIX(L.wqkv + (size_t)(c0 + sp.heads) * W, sp.heads, W);
+      if (r == "mix.g") MATRIX(L.wqkv + (size_t)L.gate_off * W, L.vd, W);
+      if (r == "mix.dt_bias") VECTOR(L.dt_bias, sp.heads);
+    }
     if (r == "mix.a1") MATRIX(L.wqkv + (size_t)(c0 + sp.heads) * W, sp.decay_rank, W);
     if (r == "mix.g1") MATRIX(L.wqkv + (size_t)(c0 + sp.heads + sp.decay_rank) * W, sp.gate_rank, W);
     if (r == "mix.a2") MATRIX(L.wa2, da, sp.decay_rank);
@@ -630,6 +820,7 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
     const long long ff = sp.expert_ff, sff = sp.shared_ff;
     if (r == "mlp.router") MATRIX(L.router, sp.experts, W);
     if (r == "mlp.router.b") VECTOR(L.router_b, sp.experts);
+    if (r == "mlp.correction") VECTOR(L.router_b, sp.experts);
     if (sff) {
       if (r == "mlp.shared.gate") PAIRED(L.sgu, sff, W);  // gate | up interleaved by unit (DenseArgs::glu)
       if (r == "mlp.shared.up") PAIRED(L.sgu + W, sff, W);
@@ -661,18 +852,40 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
   TL_REQUIRE((st->got_globals & st->need_globals) == st->need_globals,
              "tl_stack_finalize: embed / head / final.norm (and their parts) missing (have mask %d of %d)", st->got_globals,
              st->need_globals);
-  for (size_t i = 0; i < st->layers.size(); ++i)
+  for (size_t i = 0; i < st->layers.size(); ++i) {
     TL_REQUIRE(st->layers[i].expect.empty(), "tl_stack_finalize: layer %d lacks %zu tensors, the first is %s", (int)i,
                st->layers[i].expect.size(), st->layers[i].expect.begin()->c_str());
+    const Layer* sd = st->layers[i].side.get();
+    TL_REQUIRE(!sd || sd->expect.empty(), "tl_stack_finalize: the second mixer of layer %d lacks %zu tensors, the first is %s", (int)i,
+               sd->expect.size(), sd->expect.begin()->c_str());
+  }
   const size_t W = st->cfg.width, C = st->chunk;
   TL_HIP(hipMalloc(&st->cache_base, st->cache_bytes));
   float* p = static_cast<float*>(st->cache_base);
-  for (Layer& L : st->layers) {
+  for (Layer& L0 : st->layers) {
+    if (st->cfg.canon_taps > 1) {
+      L0.canon_hist1 = p;
+      p += (size_t)(st->cfg.canon_taps - 1) * W;
+      if (L0.sp.mlp != TL_MLP_NONE) {
+        L0.canon_hist2 = p;
+        p += (size_t)(st->cfg.canon_taps - 1) * W;
+      }
+    }
+   for (Layer* Lp : {&L0, L0.side.get()}) {
+    if (!Lp) continue;
+    Layer& L = *Lp;
     if (L.sp.mixer == TL_MIXER_SWA) {
       L.kc = p;
       p += (size_t)st->cfg.max_positions * L.kd;
       L.vc = p;
       p += (size_t)st->cfg.max_positions * L.vd;
+      if (L.sp.qkv_conv > 1) {
+        L.hist = p;
+        p += (size_t)(L.sp.qkv_conv - 1) * (L.qd + L.kd + L.vd);
+      }
+    } else if (L.sp.mixer == TL_MIXER_LINEAR) {
+      L.state = p;
+      p += (size_t)L.sp.heads * L.sp.vdim * L.sp.dim;
     } else if (L.sp.mixer == TL_MIXER_LATENT) {
       if (L.kd) {
         L.ckv = p;
@@ -689,7 +902,13 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
       L.hist = p;
       p += (size_t)(L.sp.conv_taps - 1) * (L.qd + L.kd + L.vd);
     }
+   }
   }
+  TL_REQUIRE((size_t)(p - static_cast<float*>(st->cache_base)) * sizeof(float) == st->cache_bytes,
+             "tl_stack_finalize: the cache layout does not add up to its allocation");
+  if (st->any_maps) TL_TRY(dev_alloc(st, &st->att2, C * st->max_od));
+  if (st->any_pair) TL_TRY(dev_alloc(st, &st->proj2, C * W));
+  if (st->cfg.canon_taps > 0) TL_TRY(dev_alloc(st, &st->hn, C * W));
   TL_TRY(dev_alloc(st, &st->x, C * W));
   TL_TRY(dev_alloc(st, &st->h, C * W));
   TL_TRY(dev_alloc(st, &st->qkv, C * st->max_qkv));
@@ -724,8 +943,14 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
   }
   {
     size_t ws = 1;
-    for (const Layer& L : st->layers)
+    std::vector<const Layer*> mixers;
+    for (const Layer& L : st->layers) {
+      mixers.push_back(&L);
+      if (L.side) mixers.push_back(L.side.get());
+    }
+    for (const Layer* Lp : mixers)
       for (int T = 1; T <= 4; ++T) {
+        const Layer& L = *Lp;
         if (L.sp.mixer != TL_MIXER_SWA && L.sp.mixer != TL_MIXER_LATENT) continue;
         const bool lat = L.sp.mixer == TL_MIXER_LATENT;
         const size_t n = tl_swa_ws_floats(T, L.sp.heads, lat ? L.sp.kv_rank : L.sp.vdim,
@@ -802,8 +1027,18 @@ void tl_stack_set_layer_hook(TlStack* st, tl_stack_layer_hook hook, void* ctx) {
 int tl_stack_cache_ptr(TlStack* st, int which, int layer, void** out) {
   TL_REQUIRE(st && st->finalized && out, "tl_stack_cache_ptr: model not finalized");
   TL_REQUIRE(layer >= 0 && layer < (int)st->layers.size(), "tl_stack_cache_ptr: layer %d out of range", layer);
-  const Layer& L = st->layers[layer];
-  // attention: 0 keys, 1 values; delta rule: 0 the state S [heads][vdim][dim], 1 the convolution's history
+  const Layer* Lp = &st->layers[layer];
+  if (which >= 4) {  // 4, 5: what 0, 1 are for the second mixer of a pair
+    TL_REQUIRE(Lp->side, "tl_stack_cache_ptr: layer %d has one mixer", layer);
+    Lp = Lp->side.get();
+    which -= 4;
+  }
+  if (which == 2 || which == 3) {  // the histories of the convolutions on what the two sublayers read
+    *out = which == 2 ? st->layers[layer].canon_hist1 : st->layers[layer].canon_hist2;
+    return 0;
+  }
+  const Layer& L = *Lp;
+  // attention: 0 keys, 1 values; delta rule and linear attention: 0 the state S [heads][vdim][dim], 1 the convolution's history
   // latent attention: 0 the rows [max_pos][kv_rank + rot_dim] this layer reads; generalized delta rule: 0 the state
   if (L.sp.mixer == TL_MIXER_SWA) *out = which == 0 ? L.kc : L.vc;
   else if (L.sp.mixer == TL_MIXER_LATENT) *out = L.ckv;
@@ -814,7 +1049,14 @@ int tl_stack_cache_ptr(TlStack* st, int which, int layer, void** out) {
 void tl_stack_bytes_per_token(const TlStack* st, int pos, double* weight_bytes, double* kv_bytes) {
   const double W = st->cfg.width;
   double wb = 2.0 * W /*embedding row*/ + 2.0 * W * st->cfg.vocab, kb = 0.0;
+  std::vector<const Layer*> mixers;
   for (const Layer& L : st->layers) {
+    mixers.push_back(&L);
+    if (L.side) mixers.push_back(L.side.get());
+    if (st->cfg.canon_taps > 0) wb += 2.0 * W * st->cfg.canon_taps * (L.sp.mlp != TL_MLP_NONE ? 2 : 1);
+  }
+  for (const Layer* Lp : mixers) {
+    const Layer& L = *Lp;
     const tl_layer_spec& sp = L.sp;
     wb += 2.0 * W * (L.pd + L.od);
     if (sp.mlp == TL_MLP_UNIT) wb += 2.0 * W * 2.0 * sp.shared_ff;
@@ -831,7 +1073,7 @@ void tl_stack_bytes_per_token(const TlStack* st, int pos, double* weight_bytes, 
     if (sp.mlp == TL_MLP_MOE)
       wb += 2.0 * W * (sp.experts + 3.0 * sp.expert_ff * sp.top + 3.0 * sp.shared_ff + (sp.shared_gate ? 1.0 : 0.0));
     if (sp.mlp == TL_MLP_DENSE) wb += 2.0 * W * 3.0 * sp.shared_ff;
-    if (sp.mixer == TL_MIXER_DELTA) {
+    if (sp.mixer == TL_MIXER_DELTA || sp.mixer == TL_MIXER_LINEAR) {
       wb += 2.0 * ((double)sp.heads * sp.dim * sp.decay_rank + (double)L.vd * sp.gate_rank);
       kb += 2.0 * 4.0 * sp.heads * sp.vdim * sp.dim;  // the state is read and written
     } else {
@@ -897,6 +1139,7 @@ int moe_experts(TlStack* st, const Layer& L, const Layer& Wt, const float* in, i
     d.slimit = sp.shared_limit;
     d.alpha = sp.act_alpha;
     d.up_add = sp.glu_up_add;
+    d.glu_kind = sp.glu;
     d.sgate = sp.shared_gate ? st->sgate : nullptr;
     d.act = st->act_buf;
     d.y = one_token_out;
@@ -921,6 +1164,7 @@ int moe_experts(TlStack* st, const Layer& L, const Layer& Wt, const float* in, i
   g.glu_limit = sp.expert_limit;
   g.glu_alpha = sp.act_alpha;
   g.glu_up_add = sp.glu_up_add;
+  g.glu_kind = sp.glu;
   TL_TRY(tl_launch_dense_gemm(g, s));
   DenseArgs d = {};  // down: item p writes the row of its slot, so that a token's choices lie side by side
   d.w = Wt.down;
@@ -951,6 +1195,7 @@ int moe_experts(TlStack* st, const Layer& L, const Layer& Wt, const float* in, i
     u.glu_limit = sp.shared_limit;
     u.glu_alpha = sp.act_alpha;
     u.glu_up_add = sp.glu_up_add;
+    u.glu_kind = sp.glu;
     TL_TRY(tl_launch_dense_gemm(u, s));
     TL_TRY(project(st, Wt.sdown, W, sff, st->sact, sff, st->sout, W, T, s));
   }
@@ -970,6 +1215,7 @@ RouterArgs router_args(TlStack* st, const Layer& L, const Layer& Wt, const float
   r.ids = st->ids;
   r.wts = st->wts;
   r.kind = sp.route;
+  r.corr = sp.route == TL_ROUTE_SIGMOID_GROUPS ? Wt.router_b : nullptr;
   r.groups = sp.route_groups;
   r.keep = sp.route_keep;
   if (sp.shared_gate) {
@@ -1005,12 +1251,32 @@ int moe_layer(TlStack* st, Layer& L, int T, hipStream_t s) {
   return tl_launch_resid_norm(n, s);
 }
 
-// ---- mixers: both read `in` [T][W] and leave their output in st->proj [T][W] ----
-int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, int start_pos, const int* pos_dev, hipStream_t s) {
+// ---- mixers: all read `in` [T][W] and leave their output in `out` [T][W] (st->proj unless the caller names another) ----
+int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, int start_pos, const int* pos_dev, hipStream_t s,
+              float* out = nullptr) {
   const tl_layer_spec& sp = L.sp;
   const tl_stack_config& c = st->cfg;
-  const int W = c.width, ld = L.pd;
+  const int W = c.width;
+  int ld = L.pd;
+  float* qkv = st->qkv;
+  if (!out) out = st->proj;
   TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));
+  if (sp.qkv_conv > 0) {  // q | k | v (+ their biases) through a convolution over time; the rest of the row is not touched
+    ConvArgs cv = {};
+    cv.in = st->qkv;
+    cv.ldi = ld;
+    cv.C = L.qd + L.kd + L.vd;
+    cv.taps = sp.qkv_conv;
+    cv.T = T;
+    cv.bias = sp.qkv_bias ? Wt.qkv_b : nullptr;
+    cv.w = Wt.conv;
+    cv.hist = L.hist;
+    cv.out = st->dq;
+    cv.ldo = cv.C;
+    TL_TRY(tl_launch_causal_conv(cv, s));
+    qkv = st->dq;
+    ld = cv.C;
+  }
   if (L.rotary_path) {
     RotaryArgs r = {};
     r.qk = st->qkv;
@@ -1037,13 +1303,15 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
     TL_TRY(tl_launch_rotary(r, s));
   } else {
     QkvPostArgs q = {};
-    q.qkv = st->qkv;
+    q.qkv = qkv;
     q.ld = ld;
     q.qd = L.qd;
     q.kd = L.kd;
     q.vd = L.vd;
-    q.q_norm = sp.qk_norm == TL_QK_NORM_WHOLE ? Wt.q_norm : nullptr;
-    q.k_norm = sp.qk_norm == TL_QK_NORM_WHOLE ? Wt.k_norm : nullptr;
+    const bool normed = sp.qk_norm == TL_QK_NORM_WHOLE || sp.qk_norm == TL_QK_NORM_HEAD_RMS;
+    q.q_norm = normed ? Wt.q_norm : nullptr;
+    q.k_norm = normed ? Wt.k_norm : nullptr;
+    q.head_dim = sp.qk_norm == TL_QK_NORM_HEAD_RMS ? sp.dim : 0;
     q.eps = c.norm_eps;
     q.kc = L.kc;
     q.vc = L.vc;
@@ -1058,7 +1326,7 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
     TL_TRY(tl_launch_qkv_post(q, s));
   }
   SwaArgs a = {};
-  a.q = st->qkv;
+  a.q = qkv;
   a.ldq = ld;
   a.kc = L.kc;
   a.vc = L.vc;
@@ -1074,26 +1342,59 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
   a.pos_dev = pos_dev;
   a.keep_first = sp.keep_first;
   a.sigmoid = sp.attn_weight == TL_ATTN_SIGMOID;
-  a.sink = sp.attn_weight == TL_ATTN_SOFTMAX_SINK;
+  a.sink = sp.attn_weight == TL_ATTN_SOFTMAX_SINK || sp.attn_weight == TL_ATTN_SOFTMAX_LEARNED_SINK;
+  a.sink_val = sp.attn_weight == TL_ATTN_SOFTMAX_LEARNED_SINK ? Wt.sinkv : nullptr;
   a.head_bias = a.sigmoid ? Wt.pb : nullptr;
+  a.softcap = sp.score_softcap;
+  a.dist_r1 = sp.dist_bias ? Wt.r1 : nullptr;
+  a.dist_r2 = sp.dist_bias ? Wt.r2 : nullptr;
   a.nsplit = tl_swa_splits(T, sp.window, c.max_positions, sp.keep_first);
   a.ws = st->swa_ws;
   a.done_cnt = st->swa_cnt;
-  TL_TRY(tl_launch_swa(a, s));
-  return project(st, Wt.wo, W, L.od, st->att, L.od, st->proj, W, T, s);
+  if (sp.score_maps == 2) {
+    // two score maps per head over the same values: q and k rows hold [map 1 | map 2] per head, so each map is a launch over
+    // every second block of dim; then o = (a1 - lambda a2) / rms (1 - diff_init) sigmoid(gate)
+    a.q_hstride = a.k_hstride = 2 * sp.dim;
+    TL_TRY(tl_launch_swa(a, s));
+    a.q = qkv + sp.dim;
+    a.kc = L.kc + sp.dim;
+    a.kld = L.kd;
+    a.out = st->att2;
+    TL_TRY(tl_launch_swa(a, s));
+    HeadNormArgs hn = {};
+    hn.o = st->att;
+    hn.sub = st->att2;
+    hn.sub_coef = Wt.lam;
+    hn.gate = sp.out_gate ? st->qkv + L.gate_off : nullptr;
+    hn.gate_ld = L.pd;
+    hn.out_scale = 1.0f - sp.diff_init;
+    hn.T = T;
+    hn.heads = sp.heads;
+    hn.vdim = sp.vdim;
+    hn.eps = c.norm_eps;
+    TL_TRY(tl_launch_head_norm(hn, s));
+  } else {
+    TL_TRY(tl_launch_swa(a, s));
+  }
+  return project(st, Wt.wo, W, L.od, st->att, L.od, out, W, T, s);
 }
 
-int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s) {
+int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s, float* out = nullptr) {
   const tl_layer_spec& sp = L.sp;
   const int W = st->cfg.width, ld = L.pd, dc = L.qd + L.kd + L.vd, da = sp.heads * sp.dim;
-  TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));  // q | k | v | beta | a1 | g1
+  if (!out) out = st->proj;
+  TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));  // q | k | v | beta | a1 | g1  (or | a | gate)
   const float* a1 = st->qkv + dc + sp.heads;
-  TL_TRY(project(st, Wt.wa2, da, sp.decay_rank, a1, ld, st->da, da, T, s));
-  TL_TRY(project(st, Wt.wg2, L.vd, sp.gate_rank, a1 + sp.decay_rank, ld, st->dg, L.vd, T, s));
+  if (!sp.decay_per_head) {
+    TL_TRY(project(st, Wt.wa2, da, sp.decay_rank, a1, ld, st->da, da, T, s));
+    TL_TRY(project(st, Wt.wg2, L.vd, sp.gate_rank, a1 + sp.decay_rank, ld, st->dg, L.vd, T, s));
+  }
   DeltaPreArgs p = {};
   p.p = st->qkv;
   p.ld = ld;
-  p.a = st->da;
+  p.a = sp.decay_per_head ? a1 : st->da;
+  p.a_per_head = sp.decay_per_head;
+  p.a_ld = ld;
   p.T = T;
   p.heads = sp.heads;
   p.kv_heads = sp.kv_heads;
@@ -1124,8 +1425,67 @@ int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, 
   d.dim = sp.dim;
   d.vdim = sp.vdim;
   TL_TRY(tl_launch_delta_scan(d, s));
-  TL_TRY(tl_launch_gated_head_norm(st->att, st->dg, Wt.onorm, T, sp.heads, sp.vdim, st->cfg.norm_eps, s));
-  return project(st, Wt.wo, W, L.od, st->att, L.od, st->proj, W, T, s);
+  if (sp.decay_per_head) {  // the gate is a direct projection and passes silu
+    HeadNormArgs hn = {};
+    hn.o = st->att;
+    hn.gate = st->qkv + L.gate_off;
+    hn.gate_ld = ld;
+    hn.gate_act = 1;
+    hn.w = Wt.onorm;
+    hn.T = T;
+    hn.heads = sp.heads;
+    hn.vdim = sp.vdim;
+    hn.eps = st->cfg.norm_eps;
+    TL_TRY(tl_launch_head_norm(hn, s));
+  } else {
+    TL_TRY(tl_launch_gated_head_norm(st->att, st->dg, Wt.onorm, T, sp.heads, sp.vdim, st->cfg.norm_eps, s));
+  }
+  return project(st, Wt.wo, W, L.od, st->att, L.od, out, W, T, s);
+}
+
+// gated linear attention: q | f | v = W h in one product; silu, the forget gate and what it writes (linear_pre); the delta
+// rule's scan without its removal step, k = 1 - f, decay = f; RMS norm per head; W_o
+int linear_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s, float* out = nullptr) {
+  const tl_layer_spec& sp = L.sp;
+  const int W = st->cfg.width, ld = L.pd, hd = sp.heads * sp.dim;
+  if (!out) out = st->proj;
+  TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));
+  LinearPreArgs p = {};
+  p.p = st->qkv;
+  p.ld = ld;
+  p.T = T;
+  p.heads = sp.heads;
+  p.dim = sp.dim;
+  p.lower = Wt.lower;
+  p.f_bias = Wt.f_bias;
+  p.qk = st->dq;
+  p.g = st->ddecay;
+  TL_TRY(tl_launch_linear_pre(p, s));
+  DeltaScanArgs d = {};
+  d.q = st->dq;
+  d.k = st->dq + hd;
+  d.ldq = 2 * hd;
+  d.v = st->qkv + 2 * hd;
+  d.ldv = ld;
+  d.g = st->ddecay;
+  d.state = L.state;
+  d.o = st->att;
+  d.T = T;
+  d.heads = sp.heads;
+  d.kv_heads = sp.heads;
+  d.dim = sp.dim;
+  d.vdim = sp.vdim;
+  d.plain_write = 1;
+  TL_TRY(tl_launch_delta_scan(d, s));
+  HeadNormArgs hn = {};
+  hn.o = st->att;
+  hn.w = Wt.onorm;
+  hn.T = T;
+  hn.heads = sp.heads;
+  hn.vdim = sp.vdim;
+  hn.eps = st->cfg.norm_eps;
+  TL_TRY(tl_launch_head_norm(hn, s));
+  return project(st, Wt.wo, W, L.od, st->att, L.od, out, W, T, s);
 }
 
 // one product per head: y[t][n * y_stride ..] = W[n] x[t][n * x_stride ..]
@@ -1308,25 +1668,151 @@ int gdelta_mixer(TlStack* st, Layer& L, const float* in, int T, hipStream_t s) {
 
 LnParams ln1_of_layer(const Layer& Wt) { return LnParams{Wt.norm1, Wt.norm1_b}; }
 
-// h = norm1(x) is already in st->h. x += mixer(h); then, with a feed-forward, h = norm2(x), x += ff(h). The launch that
-// finishes x writes the norm of the next layer's first sublayer into st->h.
+// The launch(es) that finish x in a pre-norm block: x += a_scale a + b_scale b + sum_j slot_w[j] slots[j], and the input of
+// whatever reads x next -- sublayer `which` (1: the mixer, 2: the feed-forward) of layer `next`, or nothing (next == NULL) --
+// into st->h: its norm and, where the model has one, the convolution over time on top of it (whose history is the reading
+// layer's own state, also when it borrows its tensors).
+struct Addends {
+  const float* a = nullptr;
+  float a_scale = 1.0f;
+  const float* b = nullptr;
+  float b_scale = 1.0f;
+  const float* slots = nullptr;
+  const float* slot_w = nullptr;
+  int top = 0;
+};
+int finish_x(TlStack* st, const Addends& add, Layer* next, int which, int T, hipStream_t s) {
+  const tl_stack_config& c = st->cfg;
+  const int W = c.width;
+  const Layer* Wn = next ? &st->layers[next->wsrc] : nullptr;
+  if (c.norm == TL_NORM_LAYER) {
+    TL_REQUIRE(add.a && !add.b && !add.slots && add.a_scale == 1.0f, "layer-list engine: a layer-norm block adds one sublayer output");
+    LnParams n = {};
+    if (Wn) n = which == 1 ? ln1_of_layer(*Wn) : LnParams{Wn->norm2, Wn->norm2_b};
+    return tl_launch_resid_ln(st->x, add.a, T, W, n, c.norm_eps, st->h, s);
+  }
+  const bool canon = c.canon_taps > 0 && Wn;
+  ResidRmsArgs r = {};
+  r.x = st->x;
+  r.T = T;
+  r.width = W;
+  r.a = add.a;
+  r.a_scale = add.a_scale;
+  r.b = add.b;
+  r.b_scale = add.b_scale;
+  r.slots = add.slots;
+  r.slot_w = add.slot_w;
+  r.top = add.top;
+  r.w = Wn ? (which == 1 ? Wn->norm1 : Wn->norm2) : nullptr;
+  r.eps = c.norm_eps;
+  r.h = canon ? st->hn : st->h;
+  if (r.w || r.a || r.b || r.slots) TL_TRY(tl_launch_resid_rms(r, s));
+  if (!canon) return 0;
+  ConvArgs cv = {};
+  cv.in = st->hn;
+  cv.ldi = W;
+  cv.C = W;
+  cv.taps = c.canon_taps;
+  cv.T = T;
+  cv.w = which == 1 ? Wn->canon1 : Wn->canon2;
+  cv.hist = which == 1 ? next->canon_hist1 : next->canon_hist2;
+  cv.add_input = 1;
+  cv.out = st->h;
+  cv.ldo = W;
+  return tl_launch_causal_conv(cv, s);
+}
+
+int run_mixer(TlStack* st, Layer& L, const Layer& Wt, int T, int start_pos, const int* pos_dev, hipStream_t s, float* out) {
+  switch (L.sp.mixer) {
+    case TL_MIXER_SWA: return swa_mixer(st, L, Wt, st->h, T, start_pos, pos_dev, s, out);
+    case TL_MIXER_LATENT: return latent_mixer(st, L, st->h, T, start_pos, pos_dev, s);
+    case TL_MIXER_GDELTA: return gdelta_mixer(st, L, st->h, T, s);
+    case TL_MIXER_LINEAR: return linear_mixer(st, L, Wt, st->h, T, s, out);
+    default: return delta_mixer(st, L, Wt, st->h, T, s, out);
+  }
+}
+
+// one gated unit on the rows of `in`: W_down unit(W_gate in, W_up in) -> st->sout
+int dense_unit(TlStack* st, const Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s) {
+  const tl_layer_spec& sp = L.sp;
+  const int W = st->cfg.width, ff = sp.shared_ff;
+  if (T == 1 && st->gemv_decode) {
+    MoeDecodeArgs d = {};  // the one gated unit runs where a shared expert would
+    d.x = in;
+    d.width = W;
+    d.sgu = Wt.sgu;
+    d.sdown = Wt.sdown;
+    d.sff = ff;
+    d.slimit = sp.shared_limit;
+    d.alpha = sp.act_alpha;
+    d.up_add = sp.glu_up_add;
+    d.glu_kind = sp.glu;
+    d.act = st->act_buf;
+    d.y = st->sout;
+    return tl_launch_moe_decode(d, s);
+  }
+  DenseArgs u = {};
+  u.w = Wt.sgu;
+  u.rows = 2 * ff;
+  u.cols = W;
+  u.x = in;
+  u.ldx = W;
+  u.y = st->sact;
+  u.ldy = ff;
+  u.T = T;
+  u.terms = terms_for(st, T);
+  u.glu = 1;
+  u.glu_limit = sp.shared_limit;
+  u.glu_alpha = sp.act_alpha;
+  u.glu_up_add = sp.glu_up_add;
+  u.glu_kind = sp.glu;
+  TL_TRY(tl_launch_dense_gemm(u, s));
+  return project(st, Wt.sdown, W, ff, st->sact, ff, st->sout, W, T, s);
+}
+
+// h = the input of the mixer is already in st->h. x += mixer(h) (two mixers side by side: the weighted sum of both); then,
+// with a feed-forward, h = its input from the new x, x += ff(h). The launch that finishes x prepares the input of whatever
+// reads it next.
 int pre_norm_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_dev, hipStream_t s) {
   Layer& L = st->layers[li];
   const Layer& Wt = st->layers[L.wsrc];
   const tl_layer_spec& sp = L.sp;
   const tl_stack_config& c = st->cfg;
   const int W = c.width;
-  if (sp.mixer == TL_MIXER_SWA) TL_TRY(swa_mixer(st, L, Wt, st->h, T, start_pos, pos_dev, s));
-  else if (sp.mixer == TL_MIXER_LATENT) TL_TRY(latent_mixer(st, L, st->h, T, start_pos, pos_dev, s));
-  else TL_TRY(gdelta_mixer(st, L, st->h, T, s));
-  LnParams next = {};
-  if (li + 1 < st->layers.size()) next = ln1_of_layer(st->layers[st->layers[li + 1].wsrc]);
-  if (sp.mlp == TL_MLP_NONE) return tl_launch_resid_ln(st->x, st->proj, T, W, next, c.norm_eps, st->h, s);
-  TL_TRY(tl_launch_resid_ln(st->x, st->proj, T, W, LnParams{Wt.norm2, Wt.norm2_b}, c.norm_eps, st->h, s));
-  const int ff = sp.shared_ff;
-  TL_TRY(project_act(st, Wt.sgu, ff, W, st->h, W, st->sact, ff, T, sp.act, 0, Wt.act_p, Wt.act_q, s));
-  TL_TRY(project(st, Wt.sdown, W, ff, st->sact, ff, st->sout, W, T, s));
-  return tl_launch_resid_ln(st->x, st->sout, T, W, next, c.norm_eps, st->h, s);
+  Layer* after = li + 1 < st->layers.size() ? &st->layers[li + 1] : nullptr;
+  Addends mix;
+  mix.a = st->proj;
+  TL_TRY(run_mixer(st, L, Wt, T, start_pos, pos_dev, s, st->proj));
+  if (L.side) {
+    TL_TRY(run_mixer(st, *L.side, *Wt.side, T, start_pos, pos_dev, s, st->proj2));
+    mix.a_scale = sp.mix_scale;
+    mix.b = st->proj2;
+    mix.b_scale = sp.side_scale;
+  }
+  if (sp.mlp == TL_MLP_NONE) return finish_x(st, mix, after, 1, T, s);
+  TL_TRY(finish_x(st, mix, &L, 2, T, s));
+  Addends ffo;
+  if (sp.mlp == TL_MLP_UNIT) {
+    const int ff = sp.shared_ff;
+    TL_TRY(project_act(st, Wt.sgu, ff, W, st->h, W, st->sact, ff, T, sp.act, 0, Wt.act_p, Wt.act_q, s));
+    TL_TRY(project(st, Wt.sdown, W, ff, st->sact, ff, st->sout, W, T, s));
+    ffo.a = st->sout;
+  } else if (sp.mlp == TL_MLP_DENSE) {
+    TL_TRY(dense_unit(st, L, Wt, st->h, T, s));
+    ffo.a = st->sout;
+  } else {
+    TL_TRY(tl_launch_router(router_args(st, L, Wt, st->h, T), s));
+    TL_TRY(moe_experts(st, L, Wt, st->h, T, st->sout, s));
+    if (T == 1 && st->gemv_decode) {
+      ffo.a = st->sout;  // experts (and a shared expert) already summed with the router weights
+    } else {
+      ffo.slots = st->eout;
+      ffo.slot_w = st->wts;
+      ffo.top = sp.top;
+      if (sp.shared_ff) ffo.a = st->sout;
+    }
+  }
+  return finish_x(st, ffo, after, 1, T, s);
 }
 
 DytParams dyt_of_layer(const Layer& Wt) { return DytParams{Wt.norm1_alpha, Wt.norm1, Wt.norm1_b}; }
@@ -1364,38 +1850,7 @@ int parallel_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_
       }
     }
   } else if (sp.mlp == TL_MLP_DENSE) {
-    const int ff = sp.shared_ff;
-    if (one) {
-      MoeDecodeArgs d = {};  // the one gated unit runs where a shared expert would
-      d.x = st->h;
-      d.width = W;
-      d.sgu = Wt.sgu;
-      d.sdown = Wt.sdown;
-      d.sff = ff;
-      d.slimit = sp.shared_limit;
-      d.alpha = sp.act_alpha;
-      d.up_add = sp.glu_up_add;
-      d.act = st->act_buf;
-      d.y = st->sout;
-      TL_TRY(tl_launch_moe_decode(d, fs));
-    } else {
-      DenseArgs u = {};
-      u.w = Wt.sgu;
-      u.rows = 2 * ff;
-      u.cols = W;
-      u.x = st->h;
-      u.ldx = W;
-      u.y = st->sact;
-      u.ldy = ff;
-      u.T = T;
-      u.terms = terms_for(st, T);
-      u.glu = 1;
-      u.glu_limit = sp.shared_limit;
-      u.glu_alpha = sp.act_alpha;
-      u.glu_up_add = sp.glu_up_add;
-      TL_TRY(tl_launch_dense_gemm(u, fs));
-      TL_TRY(project(st, Wt.sdown, W, ff, st->sact, ff, st->sout, W, T, fs));
-    }
+    TL_TRY(dense_unit(st, L, Wt, st->h, T, fs));
     r.b = st->sout;
   }
   if (forked) TL_HIP(hipEventRecord(st->ev_join, st->side));
@@ -1421,7 +1876,11 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
   const tl_stack_config& c = st->cfg;
   const int W = c.width;
   const bool dyt = c.norm == TL_NORM_DYT, lnorm = c.norm == TL_NORM_LAYER;
-  if (lnorm) {
+  if (c.norm == TL_NORM_RMS) {
+    TL_TRY(tl_launch_embed_rows(st->embed, c.vocab, W, tokens_dev, T, st->x, DytParams{}, st->h, s,
+                                c.embed_scale != 0.0f ? c.embed_scale : 1.0f));
+    TL_TRY(finish_x(st, Addends{}, &st->layers[0], 1, T, s));
+  } else if (lnorm) {
     const LnParams emb = c.embed_norm ? LnParams{st->embed_norm, st->embed_norm_b} : LnParams{};
     TL_TRY(tl_launch_embed_ln(st->embed, c.vocab, W, tokens_dev, T, emb, ln1_of_layer(st->layers[st->layers[0].wsrc]), c.norm_eps,
                               st->x, st->h, s));
@@ -1472,7 +1931,7 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
     TL_REQUIRE(rows_dev || n_rows == 1 || n_rows == T, "tl_stack_forward: %d rows without a list", n_rows);
     if (dyt) TL_TRY(tl_launch_dyt_rows(src, W, rows_dev, n_rows, DytParams{st->final_alpha, st->final_norm, st->final_b}, st->xn, s));
     else if (lnorm) TL_TRY(tl_launch_ln_rows(src, W, rows_dev, n_rows, LnParams{st->final_norm, st->final_b}, c.norm_eps, st->xn, s));
-    else TL_TRY(tl_launch_norm_rows(src, W, rows_dev, n_rows, st->final_norm, c.norm_eps, st->xn, s));
+    else TL_TRY(tl_launch_norm_rows(src, W, rows_dev, n_rows, st->final_norm, c.norm_eps, st->xn, s, c.norm != TL_NORM_RMS));
     TL_TRY(project(st, st->head, c.vocab, W, st->xn, W, logits_dev, c.vocab, n_rows, s, c.logit_softcap));
   }
   return 0;

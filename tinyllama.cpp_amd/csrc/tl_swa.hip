@@ -41,9 +41,10 @@ __device__ __forceinline__ void swa_merge_records(const SwaArgs& a, int t, int h
   float M = mz;
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
-  if (a.sink) M = fmaxf(M, 0.0f);
+  const float sv = a.sink && a.sink_val ? a.sink_val[h] : 0.0f;
+  if (a.sink) M = fmaxf(M, sv);
   const float fz = mz == -INFINITY ? 0.0f : expf(mz - M);
-  float L = a.sink ? expf(-M) : 0.0f;
+  float L = a.sink ? expf(sv - M) : 0.0f;
   for (int z = 0; z < a.nsplit; ++z) L += __shfl(lz * fz, z);  // in split order
   float* op = a.out + (size_t)t * a.heads * a.vdim + (size_t)h * a.vdim;
   for (int d0 = 0; d0 < a.vdim; d0 += 64) {  // every lane stays in the loop: a shuffle reads nothing from a lane that has left
@@ -83,11 +84,13 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   const int nf = a.keep_first > 0 ? (a.keep_first < jlo ? a.keep_first : jlo) : 0;
   const int pf = (nf + 63) >> 6;
   const float hb = a.sigmoid && a.head_bias ? a.head_bias[h] : 0.0f;
-  const int kld = a.kld > 0 ? a.kld : a.kv_heads * a.dim, vld = a.vld > 0 ? a.vld : a.kv_heads * a.vdim;
-  const float* qp = a.q + (size_t)t * a.ldq + (size_t)h * a.dim;
+  const int kld = a.kld > 0 ? a.kld : a.kv_heads * (a.k_hstride > 0 ? a.k_hstride : a.dim), vld = a.vld > 0 ? a.vld : a.kv_heads * a.vdim;
+  const int qhs = a.q_hstride > 0 ? a.q_hstride : a.dim, khs = a.k_hstride > 0 ? a.k_hstride : a.dim;
+  const float* qp = a.q + (size_t)t * a.ldq + (size_t)h * qhs;
+  const float r1 = a.dist_r1 ? a.dist_r1[h] : 0.0f, r2 = a.dist_r1 ? a.dist_r2[h] : 0.0f;
   for (int d = tid; d < a.dim; d += 256) qs[d] = qp[d];
   __syncthreads();
-  const bool v4 = (a.dim & 3) == 0 && (kld & 3) == 0 && ((size_t)a.kc & 15) == 0;
+  const bool v4 = (a.dim & 3) == 0 && (kld & 3) == 0 && (khs & 3) == 0 && ((size_t)a.kc & 15) == 0;
   float m = -INFINITY, l = 0.0f;
   float o[SWA_MAX_VR];
 #pragma unroll
@@ -105,7 +108,7 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
     const bool valid = j <= jend;
     float sc = -INFINITY;
     if (valid) {
-      const float* kp = a.kc + (size_t)j * kld + (size_t)g * a.dim;
+      const float* kp = a.kc + (size_t)j * kld + (size_t)g * khs;
       float acc = 0.0f;
       if (v4) {
         int d = 0;
@@ -128,6 +131,8 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
         for (int d = 0; d < a.dim; ++d) acc += qs[d] * kp[d];
       }
       sc = acc * a.scale;
+      if (a.softcap > 0.0f) sc = a.softcap * tanhf(sc / a.softcap);
+      if (a.dist_r1) sc -= r1 * log1pf(r2 * (float)(i - j));
     }
     float cm = sc;
 #pragma unroll
@@ -189,8 +194,9 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   for (int w = 0; w < SWA_WAVES; ++w) M = fmaxf(M, ml[w * 2]);
   // the sink joins where the LAST merge happens: here without splits, in swa_merge_records with them
   const bool sink_here = a.sink && nsplit == 1;
-  if (sink_here) M = fmaxf(M, 0.0f);
-  float f[SWA_WAVES], L = sink_here ? expf(-M) : 0.0f;
+  const float sv = a.sink && a.sink_val ? a.sink_val[h] : 0.0f;
+  if (sink_here) M = fmaxf(M, sv);
+  float f[SWA_WAVES], L = sink_here ? expf(sv - M) : 0.0f;
 #pragma unroll
   for (int w = 0; w < SWA_WAVES; ++w) {
     f[w] = ml[w * 2] == -INFINITY ? 0.0f : expf(ml[w * 2] - M);  // a wave without a piece counts nothing
@@ -275,7 +281,7 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   const int head = blockIdx.y, q0 = blockIdx.x * 32;
   const int g = head / (a.heads / a.kv_heads);
   const int start = a.pos_dev ? *a.pos_dev : a.start_pos;
-  const int kld = a.kld > 0 ? a.kld : a.kv_heads * a.dim, vld = a.vld > 0 ? a.vld : a.kv_heads * a.vdim;
+  const int kld = a.kld > 0 ? a.kld : a.kv_heads * (a.k_hstride > 0 ? a.k_hstride : a.dim), vld = a.vld > 0 ? a.vld : a.kv_heads * a.vdim;
   const int last_i = q0 + 31 < a.T ? q0 + 31 : a.T - 1;
   const int qpos = start + (q0 + r < a.T ? q0 + r : a.T - 1);  // rows beyond the chunk repeat its last query; never stored
   const int last_q = start + last_i;
@@ -289,13 +295,15 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   const float hb = a.sigmoid && a.head_bias ? a.head_bias[head] : 0.0f;
   // a row that no query of the tile can see (it carries weight 0) is read from a row that one of them can
   auto clamp_row = [&](int pr) { return pr > last_q ? last_q : (pr < klo && pr >= a.keep_first) ? klo : pr; };
-  const bool kvec = (a.dim & 3) == 0 && (kld & 3) == 0 && ((size_t)a.kc & 15) == 0;
+  const int qhs = a.q_hstride > 0 ? a.q_hstride : a.dim, khs = a.k_hstride > 0 ? a.k_hstride : a.dim;
+  const float r1 = a.dist_r1 ? a.dist_r1[head] : 0.0f, r2 = a.dist_r1 ? a.dist_r2[head] : 0.0f;
+  const bool kvec = (a.dim & 3) == 0 && (kld & 3) == 0 && (khs & 3) == 0 && ((size_t)a.kc & 15) == 0;
   const bool vvec = (a.vdim % DB) == 0 && (DB == 1 || (((size_t)a.vc & 15) == 0 && (DB != 3) && (vld % DB) == 0));
   // piece i (d = 8 i + 4 h + 0..3) of the lane's key row of a tile; rows outside [klo, last_q] are seen by no query of the
   // tile (masked below): their loads stay inside that range, so that nothing is read that the tile could not read
   auto load_k4 = [&](int tile, int i) -> swa_f32x4 {
     const int krow = clamp_row(tile * 32 + r);
-    const float* kp = a.kc + (size_t)krow * kld + (size_t)g * a.dim + 4 * h + 8 * i;
+    const float* kp = a.kc + (size_t)krow * kld + (size_t)g * khs + 4 * h + 8 * i;
     const int d = 8 * i + 4 * h;
     swa_f32x4 kv;
     if (kvec) {
@@ -340,7 +348,7 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   }
   for (int i = tid; i < 32 * dp; i += 256) {
     const int row = i / dp, d = i - row * dp;
-    sm_q[row * qs + d] = (q0 + row < a.T && d < a.dim) ? a.q[(size_t)(q0 + row) * a.ldq + (size_t)head * a.dim + d] : 0.0f;
+    sm_q[row * qs + d] = (q0 + row < a.T && d < a.dim) ? a.q[(size_t)(q0 + row) * a.ldq + (size_t)head * qhs + d] : 0.0f;
   }
   __syncthreads();
   swa_f32x16 o[DB];
@@ -384,7 +392,10 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
     for (int e = 0; e < 16; ++e) {
       const int p = p0 + swa_acc_row(e, h);
       const bool seen = p <= qpos && (a.window <= 0 || qpos - p < a.window || p < a.keep_first);
-      s[e] = seen ? s[e] * a.scale : -INFINITY;
+      float sc = s[e] * a.scale;
+      if (a.softcap > 0.0f) sc = a.softcap * tanhf(sc / a.softcap);
+      if (a.dist_r1) sc -= r1 * log1pf(r2 * (float)(seen ? qpos - p : 0));
+      s[e] = seen ? sc : -INFINITY;
       tmax = fmaxf(tmax, s[e]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
@@ -428,11 +439,12 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
     float M = -INFINITY;
 #pragma unroll
     for (int w = 0; w < SWA_WAVES; ++w) M = fmaxf(M, sm_m[w * 32 + r]);  // finite: every query sees itself
-    if (a.sink) M = fmaxf(M, 0.0f);
+    const float sv = a.sink && a.sink_val ? a.sink_val[head] : 0.0f;
+    if (a.sink) M = fmaxf(M, sv);
     const float mw = sm_m[wave * 32 + r];
     sm_f[wave * 32 + r] = mw == -INFINITY ? 0.0f : expf(mw - M);
     if (wave == 0) {
-      float L = a.sink ? expf(-M) : 0.0f;
+      float L = a.sink ? expf(sv - M) : 0.0f;
 #pragma unroll
       for (int w = 0; w < SWA_WAVES; ++w) {
         const float m2 = sm_m[w * 32 + r];
@@ -507,7 +519,12 @@ int tl_launch_swa(const SwaArgs& a, hipStream_t s) {
   TL_REQUIRE(a.heads <= 65535, "swa: too many heads");
   TL_REQUIRE(a.keep_first >= 0, "swa: negative number of kept first keys");
   TL_REQUIRE(!a.sink || !a.sigmoid, "swa: a sink belongs to a softmax");
-  TL_REQUIRE((a.kld == 0 || a.kld >= a.kv_heads * a.dim) && (a.vld == 0 || a.vld >= a.kv_heads * a.vdim),
+  TL_REQUIRE(!a.sink_val || a.sink, "swa: sink scores without a sink");
+  TL_REQUIRE(!a.dist_r1 == !a.dist_r2, "swa: the distance bias needs both of its vectors");
+  TL_REQUIRE(a.q_hstride >= 0 && a.k_hstride >= 0 && (a.q_hstride == 0 || a.q_hstride >= a.dim) &&
+                 (a.k_hstride == 0 || a.k_hstride >= a.dim),
+             "swa: head strides %d / %d below the key size %d", a.q_hstride, a.k_hstride, a.dim);
+  TL_REQUIRE((a.kld == 0 || a.kld >= (a.kv_heads - 1) * (a.k_hstride > 0 ? a.k_hstride : a.dim) + a.dim) && (a.vld == 0 || a.vld >= a.kv_heads * a.vdim),
              "swa: cache rows %d / %d shorter than the heads they hold", a.kld, a.vld);
   if (swa_mfma_wanted(a)) {
     switch ((a.vdim + 31) / 32) {

@@ -18,6 +18,7 @@ const std::vector<ModelFamily>& model_families() {
       {"Ralasun", "folder", load_stack_folder},
       {"Madalorn", "folder", load_stack_folder},
       {"Sogalix", "folder", load_stack_folder},
+      {"Potipel", "folder", load_stack_folder},
   };
   return table;
 }

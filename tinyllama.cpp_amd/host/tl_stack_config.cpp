@@ -28,6 +28,22 @@
 //              {"heads", "dim", "rot_dim", "vdim", "q_rank", "kv_rank", "scale", "rot": {"base", "dims"}, "kv_from": j} |
 //              {"heads", "dim"},
 //     "mlp": null | {"kind": "dense", "ff"}}]}
+// Potipel   pre-norm blocks with plain RMS norms; the embedding row is scaled; what each sublayer reads is h + conv(h), a causal
+//           convolution over time per channel (canon.taps). Mixers: "attention" = differential attention (two score maps per
+//           head over the same values, per-head q/k RMS norm, lambda from four vectors, sigmoid output gate, causal);
+//           "hgrn2" = gated linear attention whose forget gate also decides what is written; "parallel" = two mixers side by
+//           side, left a sliding-window attention (biases, a convolution on q, k, v, capped scores, a logarithmic distance
+//           bias, a learned sink per head), right the gated delta rule with one decay per head and a silu gate, summed with
+//           left_scale / right_scale. Feed-forward: a relu-gated unit, or routed experts (sigmoid scores with a correction for
+//           the choice, groups ranked by their two best, weights not normalised) of the clamped 1.702-swish form. Layers may
+//           reuse an earlier layer's tensors.
+//   {"architecture", "width", "vocab", "norm": {"eps"}, "embedding": {"scale"}, "canon": {"taps"}, "layers": [{"type":
+//     "attention" | "hgrn2" | "parallel", "weights_of": j,
+//     "mixer": {"heads", "kv_heads", "dim", "vdim", "scale", "diff"} | {"heads", "dim", "vdim"} |
+//              {"left": {"heads", "kv_heads", "dim", "vdim", "scale", "softcap", "conv", "mask": {"size"}},
+//               "right": {"heads", "kv_heads", "dim", "vdim", "conv"}, "left_scale", "right_scale"},
+//     "mlp": null | {"kind": "dense", "ff"} | {"kind": "moe", "router": {"experts", "top", "groups": {"count", "keep"}},
+//     "expert": {"ff", "limit"}}}]}
 #include <chrono>
 #include <cmath>
 #include <fstream>
@@ -241,6 +257,95 @@ tl_layer_spec sogalix_layer(const Json& layers, int index, const SafeTensorsFile
   return sp;
 }
 
+// `side` receives the second mixer of a "parallel" layer (the returned entry points at it)
+tl_layer_spec potipel_layer(const Json& layers, int index, tl_layer_spec* side) {
+  const Json& L = layers.arr[index];
+  const std::string where = "layers[" + std::to_string(index) + "]";
+  tl_layer_spec sp = {};
+  const std::string& type = L.at("type").as_string("type");
+  const Json& mx = L.at("mixer");
+  if (const Json* wo = present(L, "weights_of")) {
+    const int src = (int)wo->as_int("weights_of");
+    if (src < 0 || src >= index) throw std::runtime_error(where + ": weights_of must name an earlier layer");
+    sp.weights_of = src + 1;
+  }
+  sp.block = TL_BLOCK_PRE_NORM;
+  if (type == "attention") {
+    sp.mixer = TL_MIXER_SWA;
+    sp.heads = geti(mx, "heads");
+    sp.kv_heads = present(mx, "kv_heads") ? geti(mx, "kv_heads") : sp.heads;
+    sp.dim = geti(mx, "dim");
+    sp.vdim = present(mx, "vdim") ? geti(mx, "vdim") : sp.dim;
+    sp.scale = getf(mx, "scale");
+    sp.score_maps = 2;
+    sp.diff_init = getf(mx, "diff");
+    sp.qk_norm = TL_QK_NORM_HEAD_RMS;
+    sp.out_gate = 1;
+  } else if (type == "hgrn2") {
+    sp.mixer = TL_MIXER_LINEAR;
+    sp.heads = sp.kv_heads = geti(mx, "heads");
+    sp.dim = geti(mx, "dim");
+    sp.vdim = present(mx, "vdim") ? geti(mx, "vdim") : sp.dim;
+  } else if (type == "parallel") {
+    const Json& lt = mx.at("left");
+    sp.mixer = TL_MIXER_SWA;
+    sp.heads = geti(lt, "heads");
+    sp.kv_heads = present(lt, "kv_heads") ? geti(lt, "kv_heads") : sp.heads;
+    sp.dim = geti(lt, "dim");
+    sp.vdim = present(lt, "vdim") ? geti(lt, "vdim") : sp.dim;
+    sp.scale = getf(lt, "scale");
+    sp.score_softcap = present(lt, "softcap") ? getf(lt, "softcap") : 0.0f;
+    sp.qkv_bias = 1;
+    sp.qkv_conv = geti(lt, "conv");
+    sp.dist_bias = 1;
+    sp.attn_weight = TL_ATTN_SOFTMAX_LEARNED_SINK;
+    if (const Json* mask = present(lt, "mask")) sp.window = geti(*mask, "size");
+    const Json& rt = mx.at("right");
+    tl_layer_spec r = {};
+    r.mixer = TL_MIXER_DELTA;
+    r.heads = geti(rt, "heads");
+    r.kv_heads = present(rt, "kv_heads") ? geti(rt, "kv_heads") : r.heads;
+    r.dim = geti(rt, "dim");
+    r.vdim = present(rt, "vdim") ? geti(rt, "vdim") : r.dim;
+    r.conv_taps = geti(rt, "conv");
+    r.decay_per_head = 1;
+    r.block = TL_BLOCK_PRE_NORM;
+    *side = r;
+    sp.side = side;
+    sp.mix_scale = getf(mx, "left_scale");
+    sp.side_scale = getf(mx, "right_scale");
+  } else {
+    throw std::runtime_error(where + ": unknown layer type \"" + type + "\"");
+  }
+  if (const Json* ml = present(L, "mlp")) {
+    const std::string& kind = ml->at("kind").as_string("kind");
+    if (kind == "dense") {
+      sp.mlp = TL_MLP_DENSE;
+      sp.glu = TL_GLU_RELU;
+      sp.shared_ff = geti(*ml, "ff");
+    } else if (kind == "moe") {
+      sp.mlp = TL_MLP_MOE;
+      sp.glu = TL_GLU_SWISH;
+      sp.act_alpha = kGateAlpha;
+      sp.glu_up_add = 1.0f;
+      sp.route = TL_ROUTE_SIGMOID_GROUPS;
+      const Json& r = ml->at("router");
+      sp.experts = geti(r, "experts");
+      sp.top = geti(r, "top");
+      sp.route_groups = sp.route_keep = 1;
+      if (const Json* g = present(r, "groups")) {
+        sp.route_groups = geti(*g, "count");
+        sp.route_keep = geti(*g, "keep");
+      }
+      sp.expert_ff = geti(ml->at("expert"), "ff");
+      sp.expert_limit = getf(ml->at("expert"), "limit");
+    } else {
+      throw std::runtime_error(where + ": unknown feed-forward kind \"" + kind + "\"");
+    }
+  }
+  return sp;
+}
+
 }  // namespace
 
 void load_stack_folder(const std::string& dir, int device, int max_context, LoadedModel* out) {
@@ -253,13 +358,14 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   const Json& layers = cfg.at("layers");
   if (layers.kind != Json::ARRAY || layers.arr.empty()) throw std::runtime_error("config.json: \"layers\" is empty");
   const std::string arch = cfg.at("architecture").as_string("architecture");
-  const bool madalorn = arch == "Madalorn", sogalix = arch == "Sogalix";
+  const bool madalorn = arch == "Madalorn", sogalix = arch == "Sogalix", potipel = arch == "Potipel";
   SafeTensorsFile file;
   file.open(dir + "/model.safetensors");
-  std::vector<tl_layer_spec> specs;
+  std::vector<tl_layer_spec> specs, sides(layers.arr.size());  // (sides: second mixers, addressed by the entries of specs)
   for (size_t i = 0; i < layers.arr.size(); ++i)
     specs.push_back(madalorn  ? madalorn_layer(layers, (int)i, file)
                     : sogalix ? sogalix_layer(layers, (int)i, file)
+                    : potipel ? potipel_layer(layers, (int)i, &sides[i])
                               : ralasun_layer(layers.arr[i], (int)i, file));
   tl_stack_config sc = {};
   sc.width = geti(cfg, "width");
@@ -268,8 +374,12 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   sc.max_positions = max_context > 0 ? max_context : kDefaultContext;
   sc.norm_eps = (float)cfg.at("norm").at("eps").as_double("norm.eps");
   sc.layers = specs.data();
-  sc.norm = madalorn ? TL_NORM_DYT : sogalix ? TL_NORM_LAYER : TL_NORM_RMS_ONE_PLUS;
-  sc.embed_norm = madalorn ? 0 : 1;
+  sc.norm = madalorn ? TL_NORM_DYT : sogalix ? TL_NORM_LAYER : potipel ? TL_NORM_RMS : TL_NORM_RMS_ONE_PLUS;
+  sc.embed_norm = madalorn || potipel ? 0 : 1;
+  if (potipel) {
+    sc.embed_scale = (float)cfg.at("embedding").at("scale").as_double("embedding.scale");
+    sc.canon_taps = (int)cfg.at("canon").at("taps").as_int("canon.taps");
+  }
   if (madalorn)
     if (const Json* cap = present(cfg, "logit_softcap")) sc.logit_softcap = (float)cap->as_double("logit_softcap");
 
