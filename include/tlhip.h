@@ -458,10 +458,42 @@ int tl_general_delta(const float* p_dev, int ld, const float* dw_dev, const floa
                      float decay_scale, float* state_dev, float* o_dev, float* scratch_dev, int num_tokens, int heads, int dim,
                      void* stream);
 
+/* a causal convolution over time per channel: u[t][c] = in[t][c] (+ bias[c]); out[t][c] = act(sum_j w[c][j] u[t - taps + 1 + j][c])
+ * (+ u[t][c] with add_input); w bf16 [channels][taps], the last tap is the current token's; act 0: none, 1: silu. The inputs
+ * before this call come from history [taps - 1][channels] (oldest first, zeros for an empty sequence), which afterwards holds
+ * the last taps - 1 inputs u. out must not overlap in when num_tokens > 1. */
+int tl_causal_conv(const float* in_dev, int ld_in, int channels, int taps, int num_tokens, const float* bias_dev,
+                   const void* w_bf16_dev, float* history_dev, int act, int add_input, float* out_dev, int ld_out, void* stream);
+/* router (TL_ROUTE_SIGMOID_GROUPS): ids [T][top] best choice first, weights = the chosen experts' sigmoid scores */
+int tl_moe_route_sigmoid_groups(const float* x_dev, int num_tokens, int width, const void* w_bf16_dev,
+                                const float* correction_dev, int experts, int top, int groups, int keep, int* ids_dev,
+                                float* weights_dev, void* stream);
+/* softmax window attention with the score options of TL_MIXER_SWA: heads of a query / key row q_hstride / k_hstride floats
+ * apart (0: dim), rows ldq / k_ld / v_ld apart (0: packed); score = (q . k) scale, capped by softcap tanh(. / softcap) when
+ * softcap > 0, minus r1[head] ln(1 + r2[head] (i - j)) when r1_dev is set; sink != 0: exp(sink_dev[head]) (exp(0) without
+ * sink_dev) joins the denominator */
+int tl_window_attention_opts(const float* q_dev, int ldq, int q_hstride, const float* k_cache_dev, int k_ld, int k_hstride,
+                             const float* v_cache_dev, int v_ld, float* out_dev, int num_tokens, int start_pos, int heads,
+                             int kv_heads, int dim, int vdim, int window, float scale, float softcap, const float* r1_dev,
+                             const float* r2_dev, int sink, const float* sink_dev, void* stream);
+/* per head, in place: o <- (o - sub_coef sub) / sqrt(mean(.^2) + eps) * w * gate_fn(gate) * out_scale; sub_dev, weight_dev
+ * ([vdim], or [heads * vdim] with weight_per_head) and gate_dev (rows gate_ld apart) may be NULL; gate_act 0: sigmoid, 1: silu;
+ * out_scale 0 counts as 1 */
+int tl_head_norm(float* o_dev, const float* sub_dev, float sub_coef, const float* gate_dev, int gate_ld, int gate_act,
+                 const float* weight_dev, int weight_per_head, float out_scale, int num_tokens, int heads, int vdim, float eps,
+                 void* stream);
+/* gated linear attention (TL_MIXER_LINEAR), token by token: p [T][ld] = q | f (heads * dim each) | v (heads * vdim);
+ * q <- silu(q), f <- lower + (1 - lower) sigmoid(f + f_bias); S <- diag(f) S + (1 - f) v^T; o = S^T q. state_dev
+ * [heads][vdim][dim], updated in place; o [T][heads * vdim]; scratch_dev: 3 * T * heads * dim floats */
+int tl_gated_linear_attention(const float* p_dev, int ld, const float* lower_dev, const float* f_bias_dev, float* state_dev,
+                              float* o_dev, float* scratch_dev, int num_tokens, int heads, int dim, int vdim, void* stream);
+
 int tl_model_create_stack(const tl_stack_config* cfg, tl_model** out);
 /* tensors by checkpoint name: embed, embed.norm, final.norm, head, l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,q.norm,k.norm,vmix,pb},
  * l<i>.mix.{q,k,v}.conv, l<i>.mix.{b,a1,a2,g1,g2,A_log,dt_bias,norm}, l<i>.mlp.router, l<i>.mlp.router.b,
- * l<i>.mlp.e<j>.{gate,up,down}, l<i>.mlp.shared.{gate,up,down,sg}, l<i>.mlp.{gate,up,down,act}; latent attention
+ * l<i>.mlp.e<j>.{gate,up,down}, l<i>.mlp.shared.{gate,up,down,sg}, l<i>.mlp.{gate,up,down,act,correction}, l<i>.canon{1,2},
+ * l<i>.mix.{g,lq1,lk1,lq2,lk2,r1,r2,sink}, l<i>.mix.{q,k,v}.b, l<i>.mix.{f,f.b,lower,a}; with two mixers side by side
+ * l<i>.mix.left.* and l<i>.mix.right.*; latent attention
  * l<i>.mix.{dq,dq.norm,uq,dkv,dkv.norm,uk,uv,g,o}; generalized delta rule l<i>.mix.{r,k,v,g,a,a.b,w1,w2,w0,norm,o}; a Dynamic
  * Tanh norm <n> also has <n>.alpha and <n>.b, a layer norm <n>.b. type: TL_BF16 (matrices and vectors) or TL_F32 (vectors). */
 int tl_model_set_tensor_named(tl_model* m, const char* name, int type, const long long* shape, int ndim, const void* host_data);

@@ -203,8 +203,8 @@ class PotipelOracle:
         q, k, v = (self.conv(i, p + n, h @ w[p + n].T + w[p + n + ".b"]) for n in "qkv")
         k = self.append(i, "k", k.reshape(T, G, d))
         v = self.append(i, "v", v.reshape(T, G, vd))
-        o = softmax_attention(q.reshape(T, H, d), k, v, mx["scale"], pos, window=mx["mask"]["size"], softcap=mx["softcap"],
-                              r1=w[p + "r1"], r2=w[p + "r2"], sink=w[p + "sink"])
+        o = softmax_attention(q.reshape(T, H, d), k, v, mx["scale"], pos, window=(mx.get("mask") or {}).get("size", 0),
+                              softcap=mx.get("softcap") or 0.0, r1=w[p + "r1"], r2=w[p + "r2"], sink=w[p + "sink"])
         return o.reshape(T, -1) @ w[p + "o"].T
 
     def delta_rule(self, i, h):

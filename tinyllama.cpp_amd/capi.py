@@ -26,7 +26,10 @@ class ModelConfig(C.Structure):
 
 
 class LayerSpec(C.Structure):
-    _fields_ = [("mixer", C.c_int), ("heads", C.c_int), ("kv_heads", C.c_int), ("dim", C.c_int), ("vdim", C.c_int),
+    pass
+
+
+LayerSpec._fields_ = [("mixer", C.c_int), ("heads", C.c_int), ("kv_heads", C.c_int), ("dim", C.c_int), ("vdim", C.c_int),
                 ("window", C.c_int), ("scale", C.c_float), ("qk_norm", C.c_int), ("v_mix", C.c_int), ("mlp", C.c_int),
                 ("experts", C.c_int), ("top", C.c_int), ("expert_ff", C.c_int), ("expert_limit", C.c_float),
                 ("shared_ff", C.c_int), ("shared_limit", C.c_float), ("act_alpha", C.c_float),
@@ -36,13 +39,17 @@ class LayerSpec(C.Structure):
                 ("conv_taps", C.c_int), ("decay_rank", C.c_int), ("gate_rank", C.c_int), ("route", C.c_int),
                 ("route_groups", C.c_int), ("route_keep", C.c_int), ("shared_gate", C.c_int), ("q_temp_coef", C.c_float),
                 ("q_temp_every", C.c_int), ("q_rank", C.c_int), ("kv_rank", C.c_int), ("rot_dim", C.c_int),
-                ("kv_from", C.c_int), ("head_gate", C.c_int), ("decay_scale", C.c_float), ("act", C.c_int)]
+                ("kv_from", C.c_int), ("head_gate", C.c_int), ("decay_scale", C.c_float), ("act", C.c_int),
+                ("glu", C.c_int), ("score_maps", C.c_int), ("diff_init", C.c_float), ("out_gate", C.c_int),
+                ("qkv_bias", C.c_int), ("qkv_conv", C.c_int), ("score_softcap", C.c_float), ("dist_bias", C.c_int),
+                ("decay_per_head", C.c_int), ("side", C.POINTER(LayerSpec)), ("mix_scale", C.c_float),
+                ("side_scale", C.c_float)]
 
 
 class StackConfig(C.Structure):
     _fields_ = [("width", C.c_int), ("vocab", C.c_int), ("n_layers", C.c_int), ("max_positions", C.c_int),
                 ("norm_eps", C.c_float), ("layers", C.POINTER(LayerSpec)), ("norm", C.c_int), ("embed_norm", C.c_int),
-                ("logit_softcap", C.c_float)]
+                ("logit_softcap", C.c_float), ("embed_scale", C.c_float), ("canon_taps", C.c_int)]
 
 
 BF16 = 30
@@ -144,6 +151,13 @@ SIGNATURES = {
     "tl_dense_matmul_act": [_vp, C.c_int, C.c_int, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int, _vp],
     "tl_dense_matmul_heads": [_vp, C.c_int, C.c_int, C.c_int, _fp, C.c_int, C.c_int, _fp, C.c_int, C.c_int, C.c_int, C.c_int,
                               _vp],
+    "tl_causal_conv": [_fp, C.c_int, C.c_int, C.c_int, C.c_int, _fp, _vp, _fp, C.c_int, C.c_int, _fp, C.c_int, _vp],
+    "tl_moe_route_sigmoid_groups": [_fp, C.c_int, C.c_int, _vp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, _ip, _fp, _vp],
+    "tl_window_attention_opts": [_fp, C.c_int, C.c_int, _fp, C.c_int, C.c_int, _fp, C.c_int, _fp, C.c_int, C.c_int, C.c_int,
+                                 C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, _fp, _fp, C.c_int, _fp, _vp],
+    "tl_head_norm": [_fp, _fp, C.c_float, _fp, C.c_int, C.c_int, _fp, C.c_int, C.c_float, C.c_int, C.c_int, C.c_int,
+                     C.c_float, _vp],
+    "tl_gated_linear_attention": [_fp, C.c_int, _fp, _fp, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, _vp],
     "tl_general_delta": [_fp, C.c_int, _fp, _fp, _fp, C.c_float, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, _vp],
 }
 

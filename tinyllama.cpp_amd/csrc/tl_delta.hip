@@ -580,3 +580,59 @@ extern "C" int tl_delta_rule(const float* q_dev, const float* k_dev, const float
   a.vdim = vdim;
   return tl_launch_delta_scan(a, static_cast<hipStream_t>(stream));
 }
+
+extern "C" int tl_head_norm(float* o_dev, const float* sub_dev, float sub_coef, const float* gate_dev, int gate_ld, int gate_act,
+                            const float* weight_dev, int weight_per_head, float out_scale, int num_tokens, int heads, int vdim,
+                            float eps, void* stream) {
+  HeadNormArgs a = {};
+  a.o = o_dev;
+  a.sub = sub_dev;
+  a.sub_coef = sub_coef;
+  a.gate = gate_dev;
+  a.gate_ld = gate_ld;
+  a.gate_act = gate_act;
+  a.w = weight_dev;
+  a.w_per_head = weight_per_head;
+  a.out_scale = out_scale;
+  a.T = num_tokens;
+  a.heads = heads;
+  a.vdim = vdim;
+  a.eps = eps;
+  return tl_launch_head_norm(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tl_gated_linear_attention(const float* p_dev, int ld, const float* lower_dev, const float* f_bias_dev,
+                                         float* state_dev, float* o_dev, float* scratch_dev, int num_tokens, int heads, int dim,
+                                         int vdim, void* stream) {
+  TL_REQUIRE(scratch_dev && num_tokens > 0 && heads > 0 && dim > 0 && vdim > 0, "tl_gated_linear_attention: bad arguments");
+  TL_REQUIRE(ld >= 2 * heads * dim + heads * vdim, "tl_gated_linear_attention: row stride %d below q | f | v", ld);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t hd = (size_t)heads * dim;
+  LinearPreArgs p = {};
+  p.p = p_dev;
+  p.ld = ld;
+  p.T = num_tokens;
+  p.heads = heads;
+  p.dim = dim;
+  p.lower = lower_dev;
+  p.f_bias = f_bias_dev;
+  p.qk = scratch_dev;
+  p.g = scratch_dev + 2 * hd * num_tokens;
+  TL_TRY(tl_launch_linear_pre(p, s));
+  DeltaScanArgs d = {};
+  d.q = p.qk;
+  d.k = p.qk + hd;
+  d.ldq = (int)(2 * hd);
+  d.v = p_dev + 2 * hd;
+  d.ldv = ld;
+  d.g = p.g;
+  d.state = state_dev;
+  d.o = o_dev;
+  d.T = num_tokens;
+  d.heads = heads;
+  d.kv_heads = heads;
+  d.dim = dim;
+  d.vdim = vdim;
+  d.plain_write = 1;
+  return tl_launch_delta_scan(d, s);
+}

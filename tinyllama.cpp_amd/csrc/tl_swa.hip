@@ -645,3 +645,40 @@ extern "C" int tl_window_attention_rows(const float* q_dev, const float* k_cache
   }
   return tl_launch_swa(a, static_cast<hipStream_t>(stream));
 }
+
+extern "C" int tl_window_attention_opts(const float* q_dev, int ldq, int q_hstride, const float* k_cache_dev, int k_ld,
+                                        int k_hstride, const float* v_cache_dev, int v_ld, float* out_dev, int num_tokens,
+                                        int start_pos, int heads, int kv_heads, int dim, int vdim, int window, float scale,
+                                        float softcap, const float* r1_dev, const float* r2_dev, int sink,
+                                        const float* sink_dev, void* stream) {
+  SwaArgs a = {};
+  a.q = q_dev;
+  a.ldq = ldq > 0 ? ldq : heads * (q_hstride > 0 ? q_hstride : dim);
+  a.q_hstride = q_hstride;
+  a.kc = k_cache_dev;
+  a.kld = k_ld;
+  a.k_hstride = k_hstride;
+  a.vc = v_cache_dev;
+  a.vld = v_ld;
+  a.out = out_dev;
+  a.T = num_tokens;
+  a.heads = heads;
+  a.kv_heads = kv_heads;
+  a.dim = dim;
+  a.vdim = vdim;
+  a.window = window;
+  a.scale = scale;
+  a.softcap = softcap;
+  a.dist_r1 = r1_dev;
+  a.dist_r2 = r2_dev;
+  a.sink = sink;
+  a.sink_val = sink_dev;
+  a.start_pos = start_pos;
+  a.nsplit = tl_swa_splits(num_tokens, window, start_pos + num_tokens, 0);
+  if (a.nsplit > 1) {
+    void* ws = nullptr;
+    TL_TRY(tl_scratch(TL_SCRATCH_ATTN, sizeof(float) * tl_swa_ws_floats(num_tokens, heads, vdim, a.nsplit), &ws));
+    a.ws = static_cast<float*>(ws);
+  }
+  return tl_launch_swa(a, static_cast<hipStream_t>(stream));
+}

@@ -521,6 +521,42 @@ def _sogalix_spec(sp, i, L, tensors):
         sp.mlp, sp.act, sp.shared_ff = 3, 1, ml["ff"]
 
 
+def _potipel_spec(sp, i, L, sides):
+    """Fills entry i; a "parallel" layer's second mixer goes to sides[i], which the entry points at."""
+    mx, ml = L["mixer"], L.get("mlp")
+    sp.weights_of = L["weights_of"] + 1 if "weights_of" in L else 0
+    sp.block = 2
+    if L["type"] == "attention":
+        sp.mixer, sp.heads, sp.kv_heads = 0, mx["heads"], mx.get("kv_heads", mx["heads"])
+        sp.dim, sp.vdim, sp.scale = mx["dim"], mx.get("vdim", mx["dim"]), float(mx["scale"])
+        sp.score_maps, sp.diff_init, sp.qk_norm, sp.out_gate = 2, float(mx["diff"]), 3, 1
+    elif L["type"] == "hgrn2":
+        sp.mixer, sp.heads, sp.kv_heads, sp.dim, sp.vdim = 4, mx["heads"], mx["heads"], mx["dim"], mx.get("vdim", mx["dim"])
+    elif L["type"] == "parallel":
+        lt, rt = mx["left"], mx["right"]
+        sp.mixer, sp.heads, sp.kv_heads = 0, lt["heads"], lt.get("kv_heads", lt["heads"])
+        sp.dim, sp.vdim, sp.scale = lt["dim"], lt.get("vdim", lt["dim"]), float(lt["scale"])
+        sp.score_softcap, sp.qkv_bias, sp.qkv_conv, sp.dist_bias, sp.attn_weight = float(lt.get("softcap") or 0.0), 1, lt["conv"], 1, 3
+        sp.window = int((lt.get("mask") or {}).get("size", 0))
+        r = sides[i]
+        r.mixer, r.heads, r.kv_heads, r.dim, r.vdim = 1, rt["heads"], rt.get("kv_heads", rt["heads"]), rt["dim"], rt.get("vdim", rt["dim"])
+        r.conv_taps, r.decay_per_head, r.block = rt["conv"], 1, 2
+        sp.side = C.pointer(r)
+        sp.mix_scale, sp.side_scale = float(mx["left_scale"]), float(mx["right_scale"])
+    else:
+        raise ValueError(f"layer {i}: unknown type {L['type']!r}")
+    if ml is not None:
+        if ml["kind"] == "dense":
+            sp.mlp, sp.glu, sp.shared_ff = 2, 1, ml["ff"]
+        elif ml["kind"] == "moe":
+            r = ml["router"]
+            g = r.get("groups") or {"count": 1, "keep": 1}
+            sp.mlp, sp.route, sp.experts, sp.top, sp.route_groups, sp.route_keep = 1, 2, r["experts"], r["top"], g["count"], g["keep"]
+            sp.expert_ff, sp.expert_limit, sp.act_alpha, sp.glu_up_add = ml["expert"]["ff"], float(ml["expert"]["limit"]), 1.702, 1.0
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {ml['kind']!r}")
+
+
 def stack_config_struct(config, max_pos, tensors=None):
     """The ctypes form (tl_stack_config) of a layer-list configuration given as config.json's dictionary; returns
     (struct, the array it points into). The C++ host does the same from the file (host/tl_stack_config.cpp); this one
@@ -528,17 +564,22 @@ def stack_config_struct(config, max_pos, tensors=None):
     layers = config["layers"]
     arr = (capi.LayerSpec * len(layers))()
     madalorn, sogalix = config.get("architecture") == "Madalorn", config.get("architecture") == "Sogalix"
+    potipel = config.get("architecture") == "Potipel"
+    sides = (capi.LayerSpec * len(layers))()
     for i, L in enumerate(layers):
-        if madalorn:
+        if potipel:
+            _potipel_spec(arr[i], i, L, sides)
+        elif madalorn:
             _madalorn_spec(arr[i], i, L, tensors or {}, layers)
         elif sogalix:
             _sogalix_spec(arr[i], i, L, tensors or {})
         else:
             _ralasun_spec(arr[i], i, L)
     c = capi.StackConfig(config["width"], config["vocab"], len(layers), int(max_pos), float(config["norm"]["eps"]), arr,
-                         1 if madalorn else 2 if sogalix else 0, 0 if madalorn else 1,
-                         float(config.get("logit_softcap") or 0.0) if madalorn else 0.0)
-    return c, arr
+                         1 if madalorn else 2 if sogalix else 3 if potipel else 0, 0 if madalorn or potipel else 1,
+                         float(config.get("logit_softcap") or 0.0) if madalorn else 0.0,
+                         float(config["embedding"]["scale"]) if potipel else 0.0, int(config["canon"]["taps"]) if potipel else 0)
+    return c, (arr, sides)
 
 
 class StackModel(Model):

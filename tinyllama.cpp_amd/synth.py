@@ -525,6 +525,125 @@ def build_sogalix(config, seed=0, gain=1.0, decay_rank=8):
     return t
 
 
+def potipel_attention(heads, kv_heads, dim, vdim, diff=0.5, scale=None):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "diff": float(diff),
+            "scale": float(scale if scale is not None else dim ** -0.5)}
+
+
+def potipel_hgrn2(heads, dim, vdim):
+    return {"heads": heads, "dim": dim, "vdim": vdim}
+
+
+def potipel_pair(left_heads, left_kv_heads, left_dim, left_vdim, window, heads, kv_heads, dim, vdim, conv=4, right_conv=None,
+                 softcap=20.0, left_scale=1.0, right_scale=1.0, scale=None):
+    left = {"heads": left_heads, "kv_heads": left_kv_heads, "dim": left_dim, "vdim": left_vdim, "conv": conv,
+            "softcap": float(softcap), "scale": float(scale if scale is not None else left_dim ** -0.5)}
+    if window:
+        left["mask"] = {"size": int(window)}
+    right = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": right_conv or conv}
+    return {"left": left, "right": right, "left_scale": float(left_scale), "right_scale": float(right_scale)}
+
+
+def potipel_moe(experts, top, ff, groups=1, keep=1, limit=1.5):
+    return {"kind": "moe", "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}},
+            "expert": {"ff": ff, "limit": float(limit)}}
+
+
+def potipel_layer(kind, mixer, mlp=None, weights_of=None):
+    """kind: "attention" | "hgrn2" | "parallel"; mlp: None, an int (the relu-gated unit's size) or potipel_moe(...)."""
+    L = {"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": mlp} if isinstance(mlp, int) else mlp}
+    if weights_of is not None:
+        L["weights_of"] = weights_of
+    return L
+
+
+def potipel_config(width, vocab, layers, eps=1e-6, embed_scale=4.0, taps=3):
+    return {"architecture": "Potipel", "canon": {"taps": int(taps)}, "embedding": {"scale": float(embed_scale)},
+            "layers": list(layers), "norm": {"eps": float(eps)}, "vocab": int(vocab), "width": int(width)}
+
+
+def build_potipel(config, seed=0, gain=1.0):
+    """Random tensors {checkpoint name: uint16 bf16 bits} of a Potipel configuration (a layer with weights_of has none)."""
+    rng = np.random.default_rng(seed)
+    W, V, taps = config["width"], config["vocab"], config["canon"]["taps"]
+    t = {}
+
+    def mat(name, rows, cols, std=None):
+        t[name] = to_bf16(rng.standard_normal((rows, cols)).astype(np.float32) * (std or gain / np.sqrt(cols)))
+
+    def vec(name, n, centre, spread):
+        t[name] = to_bf16((centre + spread * rng.standard_normal(n)).astype(np.float32))
+
+    mat("embed", V, W, 1.0 / config["embedding"]["scale"])
+    vec("final.norm", W, 1.0, 0.1)
+    mat("head", V, W, 4.0 / np.sqrt(W))
+    for i, L in enumerate(config["layers"]):
+        if "weights_of" in L:
+            continue
+        mx, ml, p = L["mixer"], L.get("mlp"), f"l{i}."
+        vec(p + "norm1", W, 1.0, 0.1)
+        mat(p + "canon1", W, taps, 0.3)
+        if L["type"] == "attention":
+            H, G, d, dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+            mat(p + "mix.q", H * 2 * d, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.k", G * 2 * d, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.v", G * dv, W)
+            vec(p + "mix.q.norm", d, 1.5, 0.3)
+            vec(p + "mix.k.norm", d, 1.5, 0.3)
+            for n in ("lq1", "lk1", "lq2", "lk2"):
+                vec(p + "mix." + n, d, 0.0, 0.3)
+            mat(p + "mix.g", H * dv, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.o", W, H * dv)
+        elif L["type"] == "hgrn2":
+            H, d, dv = mx["heads"], mx["dim"], mx["vdim"]
+            mat(p + "mix.q", H * d, W, 2.0 / np.sqrt(W))
+            mat(p + "mix.f", H * d, W, 2.0 / np.sqrt(W))
+            vec(p + "mix.f.b", H * d, 1.0, 1.0)
+            t[p + "mix.lower"] = to_bf16(rng.uniform(0.0, 0.9, H * d).astype(np.float32))
+            mat(p + "mix.v", H * dv, W)
+            vec(p + "mix.norm", dv, 1.0, 0.1)
+            mat(p + "mix.o", W, H * dv)
+        else:
+            lt, rt, q = mx["left"], mx["right"], p + "mix.left."
+            H, G, d, dv = lt["heads"], lt["kv_heads"], lt["dim"], lt["vdim"]
+            for n, rows in (("q", H * d), ("k", G * d), ("v", G * dv)):
+                mat(q + n, rows, W, 2.0 / np.sqrt(W))
+                vec(q + n + ".b", rows, 0.0, 0.2)
+                mat(q + n + ".conv", rows, lt["conv"], 0.5)
+            t[q + "r1"] = to_bf16(rng.uniform(0.2, 1.5, H).astype(np.float32))
+            t[q + "r2"] = to_bf16(rng.uniform(0.05, 1.0, H).astype(np.float32))
+            vec(q + "sink", H, 0.0, 1.0)
+            mat(q + "o", W, H * dv)
+            q = p + "mix.right."
+            H, G, d, dv = rt["heads"], rt["kv_heads"], rt["dim"], rt["vdim"]
+            for n, rows in (("q", G * d), ("k", G * d), ("v", H * dv)):
+                mat(q + n, rows, W, 2.0 / np.sqrt(W))
+                mat(q + n + ".conv", rows, rt["conv"], 0.5)
+            mat(q + "b", H, W, 2.0 / np.sqrt(W))
+            mat(q + "a", H, W, 2.0 / np.sqrt(W))
+            vec(q + "A_log", H, -1.0, 1.0)
+            vec(q + "dt_bias", H, 0.0, 1.0)
+            vec(q + "norm", dv, 1.0, 0.1)
+            mat(q + "g", H * dv, W, 2.0 / np.sqrt(W))
+            mat(q + "o", W, H * dv)
+        if ml is not None:
+            vec(p + "norm2", W, 1.0, 0.1)
+            mat(p + "canon2", W, taps, 0.3)
+            if ml["kind"] == "dense":
+                mat(p + "mlp.gate", ml["ff"], W, 2.0 / np.sqrt(W))
+                mat(p + "mlp.up", ml["ff"], W, 2.0 / np.sqrt(W))
+                mat(p + "mlp.down", W, ml["ff"])
+            else:
+                E, ff = ml["router"]["experts"], ml["expert"]["ff"]
+                mat(p + "mlp.router", E, W, 3.0 / np.sqrt(W))
+                vec(p + "mlp.correction", E, 0.0, 0.3)
+                for e in range(E):
+                    mat(f"{p}mlp.e{e}.gate", ff, W, 2.0 / np.sqrt(W))
+                    mat(f"{p}mlp.e{e}.up", ff, W, 2.0 / np.sqrt(W))
+                    mat(f"{p}mlp.e{e}.down", W, ff)
+    return t
+
+
 def write_stack_dir(path, config, tensors):
     """config.json + model.safetensors (8-byte little-endian header length, JSON header, data) under `path`."""
     import json
