@@ -52,8 +52,9 @@ def parse():
     ap.add_argument("--prompt-len", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=8, help="layers in the CPU-baseline sample")
-    ap.add_argument("--family", default=None, choices=[None, "ralasun", "madalorn", "sogalix"],
-                    help="sogalix: prefill / decode throughput of that layer-list design at --sizes beside a Madalorn model of "
+    ap.add_argument("--family", default=None, choices=[None, "ralasun", "madalorn", "sogalix", "potipel"],
+                    help="potipel: prefill / decode throughput of that layer-list design at --sizes beside a Madalorn model of "
+                         "equal size; sogalix: prefill / decode throughput of that layer-list design at --sizes beside a Madalorn model of "
                          "equal size; madalorn: prefill / decode throughput of that layer-list design at --sizes beside a Ralasun model of "
                          "equal size (the closest existing model: same engine, bf16 weights, window attention, routed experts); "
                          "ralasun: prefill / decode throughput of the layer-list family at --sizes beside a Llama model of "
@@ -290,6 +291,72 @@ def _build_sogalix(S, engine, z, max_pos, rng, pool):
     return m, per_tok / n
 
 
+def _build_potipel(S, engine, z, max_pos, rng, pool):
+    """Two mixers side by side (window attention beside the delta rule with a decay per head), differential attention and
+    gated linear attention in turn; the feed-forward is the routed one of the size (sigmoid scores, 4 groups of which 2 stay)
+    in every second layer and a relu-gated unit with as many columns as a token activates there in the others. Three taps on
+    what the sublayers read, four on q, k, v."""
+    W, V, H, G, d, n = z["width"], z["vocab"], z["heads"], z["kv_heads"], z["dim"], z["layers"]
+    F = z["top"] * z["ff"] + z["shared_ff"]
+    moe = S.potipel_moe(z["experts"], z["top"], z["ff"], groups=4, keep=2, limit=7.0)
+    layers = []
+    for i in range(n):
+        ml = moe if i % 2 == 1 else F
+        if i % 3 == 0:
+            layers.append(S.potipel_layer("parallel", S.potipel_pair(H, G, d, d, z["window"], H, G, d, d, conv=4, softcap=30.0,
+                                                                     left_scale=1.0, right_scale=1.0), ml))
+        elif i % 3 == 1:
+            layers.append(S.potipel_layer("attention", S.potipel_attention(H, G, d, d, diff=0.5), ml))
+        else:
+            layers.append(S.potipel_layer("hgrn2", S.potipel_hgrn2(H, d, d), ml))
+    cfg = S.potipel_config(W, V, layers, embed_scale=1.0, taps=3)
+    m = engine.StackModel(cfg, max_pos)
+
+    def mat(nm, r, c, std=None):
+        m.set_tensor(nm, _pool_bf16(S, r * c, std or 1.0 / np.sqrt(c), rng, pool).reshape(r, c))
+
+    def vec(nm, k, centre, spread=0.05):
+        m.set_tensor(nm, S.to_bf16((centre + spread * rng.standard_normal(k)).astype(np.float32)))
+
+    mat("embed", V, W, 1.0), mat("head", V, W), vec("final.norm", W, 1.0)
+    per_tok = 0
+    for i, L in enumerate(layers):
+        p, ml = f"l{i}.", L["mlp"]
+        vec(p + "norm1", W, 1.0), vec(p + "norm2", W, 1.0), mat(p + "canon1", W, 3, 0.2), mat(p + "canon2", W, 3, 0.2)
+        if L["type"] == "parallel":
+            q = p + "mix.left."
+            for nm, rows in (("q", H * d), ("k", G * d), ("v", G * d)):
+                mat(q + nm, rows, W), vec(q + nm + ".b", rows, 0.0), mat(q + nm + ".conv", rows, 4, 0.5)
+            vec(q + "r1", H, 0.5, 0.1), vec(q + "r2", H, 0.5, 0.1), vec(q + "sink", H, 0.0, 0.5), mat(q + "o", W, H * d)
+            q = p + "mix.right."
+            for nm, rows in (("q", G * d), ("k", G * d), ("v", H * d)):
+                mat(q + nm, rows, W), mat(q + nm + ".conv", rows, 4, 0.5)
+            mat(q + "b", H, W), mat(q + "a", H, W), mat(q + "g", H * d, W), mat(q + "o", W, H * d)
+            vec(q + "A_log", H, -1.0, 0.3), vec(q + "dt_bias", H, -1.0, 0.3), vec(q + "norm", d, 1.0)
+            per_tok += (H * d + 2 * G * d + H * d) * W + (2 * G * d + 3 * H * d + 2 * H) * W
+        elif L["type"] == "attention":
+            mat(p + "mix.q", 2 * H * d, W), mat(p + "mix.k", 2 * G * d, W), mat(p + "mix.v", G * d, W), mat(p + "mix.g", H * d, W)
+            mat(p + "mix.o", W, H * d), vec(p + "mix.q.norm", d, 1.0), vec(p + "mix.k.norm", d, 1.0)
+            for nm in ("lq1", "lk1", "lq2", "lk2"):
+                vec(p + "mix." + nm, d, 0.0, 0.1)
+            per_tok += (2 * H * d + 3 * G * d + 2 * H * d) * W
+        else:
+            mat(p + "mix.q", H * d, W), mat(p + "mix.f", H * d, W), mat(p + "mix.v", H * d, W), mat(p + "mix.o", W, H * d)
+            vec(p + "mix.f.b", H * d, 1.0, 0.5), vec(p + "mix.norm", d, 1.0)
+            m.set_tensor(p + "mix.lower", S.to_bf16(rng.uniform(0.0, 0.9, H * d).astype(np.float32)))
+            per_tok += 4 * H * d * W
+        if isinstance(ml, dict) and ml["kind"] == "moe":
+            mat(p + "mlp.router", z["experts"], W), vec(p + "mlp.correction", z["experts"], 0.0, 0.1)
+            for e in range(z["experts"]):
+                mat(p + f"mlp.e{e}.gate", z["ff"], W), mat(p + f"mlp.e{e}.up", z["ff"], W), mat(p + f"mlp.e{e}.down", W, z["ff"])
+            per_tok += 3 * W * z["top"] * z["ff"] + W * z["experts"]
+        else:
+            mat(p + "mlp.gate", F, W), mat(p + "mlp.up", F, W), mat(p + "mlp.down", W, F)
+            per_tok += 3 * W * F
+    m.finalize()
+    return m, per_tok / n
+
+
 def stack_bench(args):
     from _pkg import load_package
     pkg = load_package()
@@ -304,6 +371,23 @@ def stack_bench(args):
         z = STACK_SIZES[name]
         W, V = z["width"], z["vocab"]
         max_pos = T + args.steps + args.warmup + 64
+        if args.family == "potipel":
+            z = dict(z, vdim=z["dim"])
+            t0 = time.time()
+            m, per_tok = _build_potipel(S, engine, z, max_pos, rng, pool)
+            r = {"size": name, "shape": z, "layers": "parallel (window attention | delta rule) / differential attention / hgrn2 in turn",
+                 "load_s": round(time.time() - t0, 1)}
+            got, toks, first = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+            r.update(got)
+            m.free()
+            if not args.no_twin:
+                m, per_tok = _build_madalorn(S, engine, z, max_pos, rng, pool)
+                tw, _, _ = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+                m.free()
+                r["madalorn_twin"] = tw
+            results.append(r)
+            print(json.dumps(r), file=sys.stderr, flush=True)
+            continue
         if args.family == "sogalix":
             z = dict(z, vdim=z["dim"])
             t0 = time.time()
@@ -379,7 +463,9 @@ def stack_bench(args):
             r["llama_twin"] = tw
         results.append(r)
         print(json.dumps(r), file=sys.stderr, flush=True)
-    label = ("layer-list family (Sogalix): prefill / decode tokens/s beside a Madalorn model of equal size"
+    label = ("layer-list family (Potipel): prefill / decode tokens/s beside a Madalorn model of equal size"
+             if args.family == "potipel" else
+             "layer-list family (Sogalix): prefill / decode tokens/s beside a Madalorn model of equal size"
              if args.family == "sogalix" else
              "layer-list family (Madalorn): prefill / decode tokens/s beside a Ralasun model of equal size"
              if args.family == "madalorn" else

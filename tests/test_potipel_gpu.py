@@ -355,7 +355,7 @@ def test_residual_stream_after_every_layer(env, variant):
     if variant in ("mixed", "wide"):
         m.set_prefill(1, 1)                                       # bf16 activations in the chunk products
         m.reset_kv()
-        assert rel_rms(m.prefill_rows(toks, 0), want) < BF16_TOL
+        assert most_rows(m.prefill_rows(toks, 0), want) < BF16_TOL
     m.free()
 
 

@@ -189,7 +189,23 @@ __global__ __launch_bounds__(1024) void resid_rms_kernel(const ResidRmsArgs a) {
   if (!a.w) return;
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)a.width + a.eps), w_add = a.one_plus ? 1.0f : 0.0f;
-  for (int c = threadIdx.x; c < a.width; c += blockDim.x) a.h[(size_t)t * a.width + c] = row[c] * inv * (w_add + a.w[c]);
+  if (!a.canon_w) {
+    for (int c = threadIdx.x; c < a.width; c += blockDim.x) a.h[(size_t)t * a.width + c] = row[c] * inv * (w_add + a.w[c]);
+    return;
+  }
+  const int H = a.canon_taps - 1;  // (one token: the launcher checks)
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+    const float cur = row[c] * inv * (w_add + a.w[c]);
+    const unsigned short* w = a.canon_w + (size_t)c * a.canon_taps;
+    float acc = tl_bf2f(w[H]) * cur;
+    for (int j = 0; j < H; ++j) {
+      const float u = a.canon_hist[(size_t)j * a.width + c];
+      acc += tl_bf2f(w[j]) * u;
+      if (j > 0) a.canon_hist[(size_t)(j - 1) * a.width + c] = u;
+    }
+    if (H > 0) a.canon_hist[(size_t)(H - 1) * a.width + c] = cur;
+    a.h[c] = cur + acc;
+  }
 }
 
 constexpr int kMaxRowFloats = 16 * 1024;  // 64 KB of LDS for the staged row
@@ -410,6 +426,8 @@ int tl_launch_resid_rms(const ResidRmsArgs& a, hipStream_t s) {
   TL_REQUIRE(a.width > 0 && a.width <= kMaxRowFloats, "resid_rms: width %d outside (0, %d]", a.width, kMaxRowFloats);
   TL_REQUIRE(!a.slots || (a.slot_w && a.top > 0), "resid_rms: expert slots without weights");
   TL_REQUIRE(!a.w || a.h, "resid_rms: a norm without its output");
+  TL_REQUIRE(!a.canon_w || (a.T == 1 && a.w && a.canon_taps >= 1 && (a.canon_taps == 1 || a.canon_hist)),
+             "resid_rms: the convolution rides along for one token behind a norm (%d tokens, %d taps)", a.T, a.canon_taps);
   resid_rms_kernel<<<a.T, row_threads(a.T), sizeof(float) * a.width, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;

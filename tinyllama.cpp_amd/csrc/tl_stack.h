@@ -186,6 +186,12 @@ struct ResidRmsArgs {
   int one_plus;
   float eps;
   float* h;              // [T][width]
+  // one token (the decode step): the convolution over time on what the sublayer reads rides in this launch --
+  // h <- h + conv(h) with canon_w bf16 [width][canon_taps] and its history [canon_taps - 1][width], which is shifted here
+  // (a thread is the only reader of its channels' history). canon_w == NULL: none
+  const uint16_t* canon_w;
+  float* canon_hist;
+  int canon_taps;
 };
 int tl_launch_resid_rms(const ResidRmsArgs& a, hipStream_t s);
 // ---- norm-first blocks: Dynamic Tanh (elementwise, no statistics) and the plain residual sum ------------------------------

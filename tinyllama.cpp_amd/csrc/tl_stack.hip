@@ -109,6 +109,7 @@ struct TlStack {
   int exact_below = 64;     // portions shorter than this always multiply with three terms (TL_STACK_EXACT_BELOW; at least 2)
   bool gemv_decode = true;
   bool fuse_router = true;  // TL_STACK_FUSE_ROUTER=0: the router as a launch of its own (A/B, tests)
+  bool fuse_canon = true;   // TL_STACK_FUSE_CANON=0: the convolution on what a sublayer reads as a launch of its own also for one token
   // One token through a parallel block: mixer and feed-forward read the same h and meet only in the residual sum, so the
   // feed-forward's launches go to a second stream (forked and joined by events; under capture they become a parallel branch
   // of the graph) and the step's critical path per layer is the longer of the two chains, not their sum. TL_STACK_FORK=0: one stream.
@@ -402,10 +403,7 @@ int setup_mixer(TlStack* st, Layer& L, int i, bool own, int* first_mix) {
       TL_TRY(dev_alloc(st, &L.onorm, sp.vdim));
     }
   }
-  if (own) {
-    TL_TRY(dev_alloc(st, &L.wqkv, (size_t)L.pd * W));
-    TL_TRY(dev_alloc(st, &L.wo, W * L.od));
-  }
+  if (own) TL_TRY(dev_alloc(st, &L.wo, W * L.od));
   st->max_qkv = L.pd > st->max_qkv ? L.pd : st->max_qkv;
   st->max_od = L.od > st->max_od ? L.od : st->max_od;
   st->max_vd = L.vd > st->max_vd ? L.vd : st->max_vd;
@@ -458,6 +456,14 @@ int setup_layer(TlStack* st, int i, int* first_mix) {
     L.side->wsrc = L.wsrc;
     TL_TRY(setup_mixer(st, *L.side, i, own, first_mix));
     st->any_pair = true;
+  }
+  {  // the first product's matrix; two mixers side by side share one, the second mixer's rows behind the first's: one product
+    const int rows = L.pd + (L.side ? L.side->pd : 0);
+    if (own) {
+      TL_TRY(dev_alloc(st, &L.wqkv, (size_t)rows * W));
+      if (L.side) L.side->wqkv = L.wqkv + (size_t)L.pd * W;
+    }
+    st->max_qkv = rows > st->max_qkv ? rows : st->max_qkv;
   }
   if (own) {
     TL_TRY(dev_alloc(st, &L.norm1, W));
@@ -595,6 +601,7 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
   if (const char* e = getenv("TL_STACK_GEMV")) st->gemv_decode = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FUSE_ROUTER")) st->fuse_router = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FORK")) st->fork = atoi(e) != 0;
+  if (const char* e = getenv("TL_STACK_FUSE_CANON")) st->fuse_canon = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_LEAD")) st->lead = atoi(e) > 0 ? atoi(e) : 0;
   if (const char* e = getenv("TL_STACK_EXACT_BELOW")) st->exact_below = atoi(e) > 2 ? atoi(e) : 2;
   if (const char* e = getenv("TL_STACK_LATENT_EXPAND")) st->latent_expand = atoi(e) > 0 ? atoi(e) : 0;
@@ -1252,18 +1259,21 @@ int moe_layer(TlStack* st, Layer& L, int T, hipStream_t s) {
 }
 
 // ---- mixers: all read `in` [T][W] and leave their output in `out` [T][W] (st->proj unless the caller names another) ----
+// pre != NULL: the first product has been done by the caller (rows pre_ld floats apart); `in` is then not read
 int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, int start_pos, const int* pos_dev, hipStream_t s,
-              float* out = nullptr) {
+              float* out = nullptr, float* pre = nullptr, int pre_ld = 0) {
   const tl_layer_spec& sp = L.sp;
   const tl_stack_config& c = st->cfg;
   const int W = c.width;
-  int ld = L.pd;
-  float* qkv = st->qkv;
+  int ld = pre ? pre_ld : L.pd;
+  float* qkv = pre ? pre : st->qkv;
+  float* const row0 = qkv;  // the product's rows (the gate columns stay there when q | k | v move on)
+  const int ld0 = ld;
   if (!out) out = st->proj;
-  TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));
+  if (!pre) TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));
   if (sp.qkv_conv > 0) {  // q | k | v (+ their biases) through a convolution over time; the rest of the row is not touched
     ConvArgs cv = {};
-    cv.in = st->qkv;
+    cv.in = qkv;
     cv.ldi = ld;
     cv.C = L.qd + L.kd + L.vd;
     cv.taps = sp.qkv_conv;
@@ -1279,7 +1289,7 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
   }
   if (L.rotary_path) {
     RotaryArgs r = {};
-    r.qk = st->qkv;
+    r.qk = qkv;
     r.ld = ld;
     r.heads = sp.heads;
     r.kv_heads = sp.kv_heads;
@@ -1293,7 +1303,7 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
     if (sp.values_are_keys) {
       r.vc = L.vc;
     } else {
-      r.v_src = st->qkv + L.qd + L.kd;
+      r.v_src = qkv + L.qd + L.kd;
       r.v_dst = L.vc;
       r.vd = L.vd;
     }
@@ -1365,8 +1375,8 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
     hn.o = st->att;
     hn.sub = st->att2;
     hn.sub_coef = Wt.lam;
-    hn.gate = sp.out_gate ? st->qkv + L.gate_off : nullptr;
-    hn.gate_ld = L.pd;
+    hn.gate = sp.out_gate ? row0 + L.gate_off : nullptr;
+    hn.gate_ld = ld0;
     hn.out_scale = 1.0f - sp.diff_init;
     hn.T = T;
     hn.heads = sp.heads;
@@ -1379,18 +1389,20 @@ int swa_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, in
   return project(st, Wt.wo, W, L.od, st->att, L.od, out, W, T, s);
 }
 
-int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s, float* out = nullptr) {
+int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s, float* out = nullptr,
+                float* pre = nullptr, int pre_ld = 0) {
   const tl_layer_spec& sp = L.sp;
-  const int W = st->cfg.width, ld = L.pd, dc = L.qd + L.kd + L.vd, da = sp.heads * sp.dim;
+  const int W = st->cfg.width, ld = pre ? pre_ld : L.pd, dc = L.qd + L.kd + L.vd, da = sp.heads * sp.dim;
+  float* const P = pre ? pre : st->qkv;
   if (!out) out = st->proj;
-  TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));  // q | k | v | beta | a1 | g1  (or | a | gate)
-  const float* a1 = st->qkv + dc + sp.heads;
+  if (!pre) TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));  // q | k | v | beta | a1 | g1  (or | a | gate)
+  const float* a1 = P + dc + sp.heads;
   if (!sp.decay_per_head) {
     TL_TRY(project(st, Wt.wa2, da, sp.decay_rank, a1, ld, st->da, da, T, s));
     TL_TRY(project(st, Wt.wg2, L.vd, sp.gate_rank, a1 + sp.decay_rank, ld, st->dg, L.vd, T, s));
   }
   DeltaPreArgs p = {};
-  p.p = st->qkv;
+  p.p = P;
   p.ld = ld;
   p.a = sp.decay_per_head ? a1 : st->da;
   p.a_per_head = sp.decay_per_head;
@@ -1428,7 +1440,7 @@ int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, 
   if (sp.decay_per_head) {  // the gate is a direct projection and passes silu
     HeadNormArgs hn = {};
     hn.o = st->att;
-    hn.gate = st->qkv + L.gate_off;
+    hn.gate = P + L.gate_off;
     hn.gate_ld = ld;
     hn.gate_act = 1;
     hn.w = Wt.onorm;
@@ -1445,13 +1457,15 @@ int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, 
 
 // gated linear attention: q | f | v = W h in one product; silu, the forget gate and what it writes (linear_pre); the delta
 // rule's scan without its removal step, k = 1 - f, decay = f; RMS norm per head; W_o
-int linear_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s, float* out = nullptr) {
+int linear_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, hipStream_t s, float* out = nullptr,
+                 float* pre = nullptr, int pre_ld = 0) {
   const tl_layer_spec& sp = L.sp;
-  const int W = st->cfg.width, ld = L.pd, hd = sp.heads * sp.dim;
+  const int W = st->cfg.width, ld = pre ? pre_ld : L.pd, hd = sp.heads * sp.dim;
+  float* const P = pre ? pre : st->qkv;
   if (!out) out = st->proj;
-  TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));
+  if (!pre) TL_TRY(project(st, Wt.wqkv, ld, W, in, W, st->qkv, ld, T, s));
   LinearPreArgs p = {};
-  p.p = st->qkv;
+  p.p = P;
   p.ld = ld;
   p.T = T;
   p.heads = sp.heads;
@@ -1465,7 +1479,7 @@ int linear_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T,
   d.q = st->dq;
   d.k = st->dq + hd;
   d.ldq = 2 * hd;
-  d.v = st->qkv + 2 * hd;
+  d.v = P + 2 * hd;
   d.ldv = ld;
   d.g = st->ddecay;
   d.state = L.state;
@@ -1706,6 +1720,13 @@ int finish_x(TlStack* st, const Addends& add, Layer* next, int which, int T, hip
   r.w = Wn ? (which == 1 ? Wn->norm1 : Wn->norm2) : nullptr;
   r.eps = c.norm_eps;
   r.h = canon ? st->hn : st->h;
+  if (canon && T == 1 && st->fuse_canon) {  // one token: norm, convolution and the shift of its history in the same launch
+    r.h = st->h;
+    r.canon_w = which == 1 ? Wn->canon1 : Wn->canon2;
+    r.canon_hist = which == 1 ? next->canon_hist1 : next->canon_hist2;
+    r.canon_taps = c.canon_taps;
+    return tl_launch_resid_rms(r, s);
+  }
   if (r.w || r.a || r.b || r.slots) TL_TRY(tl_launch_resid_rms(r, s));
   if (!canon) return 0;
   ConvArgs cv = {};
@@ -1722,13 +1743,14 @@ int finish_x(TlStack* st, const Addends& add, Layer* next, int which, int T, hip
   return tl_launch_causal_conv(cv, s);
 }
 
-int run_mixer(TlStack* st, Layer& L, const Layer& Wt, int T, int start_pos, const int* pos_dev, hipStream_t s, float* out) {
+int run_mixer(TlStack* st, Layer& L, const Layer& Wt, int T, int start_pos, const int* pos_dev, hipStream_t s, float* out,
+              float* pre = nullptr, int pre_ld = 0) {
   switch (L.sp.mixer) {
-    case TL_MIXER_SWA: return swa_mixer(st, L, Wt, st->h, T, start_pos, pos_dev, s, out);
+    case TL_MIXER_SWA: return swa_mixer(st, L, Wt, st->h, T, start_pos, pos_dev, s, out, pre, pre_ld);
     case TL_MIXER_LATENT: return latent_mixer(st, L, st->h, T, start_pos, pos_dev, s);
     case TL_MIXER_GDELTA: return gdelta_mixer(st, L, st->h, T, s);
-    case TL_MIXER_LINEAR: return linear_mixer(st, L, Wt, st->h, T, s, out);
-    default: return delta_mixer(st, L, Wt, st->h, T, s, out);
+    case TL_MIXER_LINEAR: return linear_mixer(st, L, Wt, st->h, T, s, out, pre, pre_ld);
+    default: return delta_mixer(st, L, Wt, st->h, T, s, out, pre, pre_ld);
   }
 }
 
@@ -1782,9 +1804,16 @@ int pre_norm_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_
   Layer* after = li + 1 < st->layers.size() ? &st->layers[li + 1] : nullptr;
   Addends mix;
   mix.a = st->proj;
-  TL_TRY(run_mixer(st, L, Wt, T, start_pos, pos_dev, s, st->proj));
   if (L.side) {
-    TL_TRY(run_mixer(st, *L.side, *Wt.side, T, start_pos, pos_dev, s, st->proj2));
+    // both mixers' first products as one (their matrices lie one behind the other); each then works on its columns
+    const int ld = L.pd + L.side->pd;
+    TL_TRY(project(st, Wt.wqkv, ld, W, st->h, W, st->qkv, ld, T, s));
+    TL_TRY(run_mixer(st, L, Wt, T, start_pos, pos_dev, s, st->proj, st->qkv, ld));
+    TL_TRY(run_mixer(st, *L.side, *Wt.side, T, start_pos, pos_dev, s, st->proj2, st->qkv + L.pd, ld));
+  } else {
+    TL_TRY(run_mixer(st, L, Wt, T, start_pos, pos_dev, s, st->proj, nullptr, 0));
+  }
+  if (L.side) {
     mix.a_scale = sp.mix_scale;
     mix.b = st->proj2;
     mix.b_scale = sp.side_scale;
