@@ -505,6 +505,26 @@ def test_graph_replays_match_the_eager_step(env):
     graph.free()
 
 
+def test_one_token_step_with_and_without_its_fusions(env):
+    """The one-token step as it is served (the convolution on what a sublayer reads inside the norm's launch) against the same
+    step with one launch per operation, and against the oracle."""
+    cfg = small_config(env["synth"], "mixed")
+    rng = np.random.default_rng(9)
+    toks = rng.integers(0, cfg["vocab"], 70).astype(np.int32)
+    tensors = env["synth"].build_potipel(cfg, 43)
+    served, _, orc = make(env, cfg, tensors=tensors)
+    plain, _, _ = make(env, cfg, tensors=tensors, TL_STACK_FUSE_CANON=0)
+    assert served.graph_nodes() < plain.graph_nodes()
+    want = orc.forward(list(toks))
+    for m in (served, plain):
+        m.prefill_rows(toks[:25], 0, np.array([24], np.int32))
+    a = np.stack([served.decode(int(toks[i]), i)[0] for i in range(25, 70)])
+    b = np.stack([plain.decode(int(toks[i]), i)[0] for i in range(25, 70)])
+    assert rel_rms(a, want[25:]) < FP32_TOL and rel_rms(b, want[25:]) < FP32_TOL and rel_rms(a, b) < FP32_TOL
+    served.free()
+    plain.free()
+
+
 def test_generation_through_the_host_session(env, tmp_path):
     """The framework's own entry point: a checkpoint folder opened by tlhost::Session (model registry, config.json reader,
     safetensors loader), greedy generate() for a short and a long prompt, generate_batch over unequal prompts against each

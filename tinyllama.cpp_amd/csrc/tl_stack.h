@@ -11,6 +11,7 @@
 //                 cache write, residual += norm(sublayer output), row-gathering norm in front of the head; layer norms of
 //                 pre-norm blocks (residual sum + the norm of the sublayer that follows)
 //   tl_rope.hip   rotary positions, per-head unit norm;  tl_delta.hip  two delta-rule recurrences with their preparation
+//   tl_conv.hip   a short causal convolution over time per channel with its history (sublayer inputs; projected q, k, v)
 //   tl_latent.hip latent attention: norms of the latents, the rotated shared key part, cache rows, per-head output gate
 #pragma once
 #include "tl_internal.h"

@@ -21,8 +21,18 @@
 //                         latent layer's cache (kv_from) and then projects no latent of its own
 //         TL_MIXER_GDELTA r | k | v | gate | a | w1 = W h in one product (tanh on the w1 rows in its epilogue), w2 behind w1;
 //                         gdelta_pre, gdelta_scan over a per-head state, gated head norm with weights per head; W_o
+//         TL_MIXER_LINEAR gated linear attention: q | f | v = W h in one product; silu, forget gate and what it writes (linear_pre);
+//                         the delta rule's scan without its removal step; RMS norm per head; W_o
+//         TL_MIXER_SWA with its options: two score maps per head over the same values (differential attention: one attention
+//                         launch per map, then (a1 - lambda a2) / rms (1 - diff) sigmoid(gate)), a norm per head and map, biases
+//                         and a causal convolution on q, k, v (tl_conv.hip), capped scores, a logarithmic distance bias, a learned
+//                         sink per head; TL_MIXER_DELTA with one decay per head and direct projections for decay and gate
+//         Two mixers side by side (tl_layer_spec::side): both read the same input, their first products are one product, the
+//                         layer's mixer output is mix_scale * first + side_scale * second
+//         Pre-norm blocks behind the plain RMS norm (TL_NORM_RMS) may add a causal convolution over time to what each sublayer
+//                         reads (canon_taps); the embedding row may be scaled (embed_scale)
 // Feed-forward  TL_MLP_UNIT  W_down act(W_up h), the activation in the first product's epilogue (pre-norm blocks)
-//               TL_MLP_MOE  router (two kinds, tl_moe.hip) -> top experts (gated units) + optional shared expert, optionally
+//               TL_MLP_MOE  router (three kinds, tl_moe.hip) -> top experts (gated units) + optional shared expert, optionally
 //                           gated per token;  TL_MLP_DENSE  one gated unit (it runs where a shared expert would)
 // A layer may use an earlier layer's tensors (weights_of) with a cache or state of its own.
 // The residual stream, norms, router, attention scores, caches and states are FP32; matrix operands of a prompt chunk are bf16
@@ -30,7 +40,8 @@
 //
 // Cache and state: one allocation. Attention layers: K [max_positions][kv_heads * dim] and V [max_positions][kv_heads * vdim],
 // flat by absolute position; a window only bounds what attention reads. Delta layers: S [heads][vdim][dim] and the
-// convolution's last taps - 1 inputs; latent layers with a projection of their
+// convolution's last taps - 1 inputs (linear attention: S only; attention with a convolution on q, k, v: that history too;
+// every layer: the histories of the convolutions on what its sublayers read); latent layers with a projection of their
 // own: rows [max_positions][kv_rank + rot_dim]; generalized delta layers: S [heads][dim][dim]. tl_stack_reset gives everything back (one sequence at a time): zeros are the state of
 // an empty sequence.
 #include <math.h>
