@@ -477,8 +477,7 @@ int tl_window_attention_opts(const float* q_dev, int ldq, int q_hstride, const f
                              int kv_heads, int dim, int vdim, int window, float scale, float softcap, const float* r1_dev,
                              const float* r2_dev, int sink, const float* sink_dev, void* stream);
 /* per head, in place: o <- (o - sub_coef sub) / sqrt(mean(.^2) + eps) * w * gate_fn(gate) * out_scale; sub_dev, weight_dev
- * ([vdim], or [heads * vdim] with weight_per_head) and gate_dev (rows gate_ld apart) may be NULL; gate_act 0: sigmoid, 1: silu;
- * out_scale 0 counts as 1 */
+ * ([vdim], or [heads * vdim] with weight_per_head) and gate_dev (rows gate_ld apart) may be NULL; gate_act 0: sigmoid, 1: silu */
 int tl_head_norm(float* o_dev, const float* sub_dev, float sub_coef, const float* gate_dev, int gate_ld, int gate_act,
                  const float* weight_dev, int weight_per_head, float out_scale, int num_tokens, int heads, int vdim, float eps,
                  void* stream);

@@ -506,14 +506,14 @@ def test_graph_replays_match_the_eager_step(env):
 
 
 def test_one_token_step_with_and_without_its_fusions(env):
-    """The one-token step as it is served (the convolution on what a sublayer reads inside the norm's launch) against the same
-    step with one launch per operation, and against the oracle."""
+    """The one-token step as it is served (the convolution on what a sublayer reads and the router inside the norm's launch)
+    against the same step with one launch per operation, and against the oracle."""
     cfg = small_config(env["synth"], "mixed")
     rng = np.random.default_rng(9)
     toks = rng.integers(0, cfg["vocab"], 70).astype(np.int32)
     tensors = env["synth"].build_potipel(cfg, 43)
     served, _, orc = make(env, cfg, tensors=tensors)
-    plain, _, _ = make(env, cfg, tensors=tensors, TL_STACK_FUSE_CANON=0)
+    plain, _, _ = make(env, cfg, tensors=tensors, TL_STACK_FUSE_CANON=0, TL_STACK_FUSE_ROUTER=0)
     assert served.graph_nodes() < plain.graph_nodes()
     want = orc.forward(list(toks))
     for m in (served, plain):

@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void head_norm_kernel(const HeadNormArgs a) {
   const float* sub = a.sub ? a.sub + (size_t)i * vdim : nullptr;
   const float* g = a.gate ? a.gate + (size_t)t * a.gate_ld + (size_t)h * vdim : nullptr;
   const float* wh = a.w ? a.w + (a.w_per_head ? (size_t)h * vdim : 0) : nullptr;
-  const float scale = a.out_scale != 0.0f ? a.out_scale : 1.0f;
+  const float scale = a.out_scale;
   float ss = 0.0f;
   for (int d = lane; d < vdim; d += 64) {
     const float v = sub ? x[d] - a.sub_coef * sub[d] : x[d];
@@ -437,6 +437,7 @@ int tl_launch_gated_head_norm_rows(float* o, const float* gate, int gate_ld, con
   a.gate_ld = gate_ld;
   a.w = w;
   a.w_per_head = w_per_head;
+  a.out_scale = 1.0f;
   a.T = T;
   a.heads = heads;
   a.vdim = vdim;

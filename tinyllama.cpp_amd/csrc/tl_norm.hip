@@ -190,22 +190,50 @@ __global__ __launch_bounds__(1024) void resid_rms_kernel(const ResidRmsArgs a) {
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)a.width + a.eps), w_add = a.one_plus ? 1.0f : 0.0f;
   if (!a.canon_w) {
-    for (int c = threadIdx.x; c < a.width; c += blockDim.x) a.h[(size_t)t * a.width + c] = row[c] * inv * (w_add + a.w[c]);
-    return;
-  }
-  const int H = a.canon_taps - 1;  // (one token: the launcher checks)
-  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
-    const float cur = row[c] * inv * (w_add + a.w[c]);
-    const unsigned short* w = a.canon_w + (size_t)c * a.canon_taps;
-    float acc = tl_bf2f(w[H]) * cur;
-    for (int j = 0; j < H; ++j) {
-      const float u = a.canon_hist[(size_t)j * a.width + c];
-      acc += tl_bf2f(w[j]) * u;
-      if (j > 0) a.canon_hist[(size_t)(j - 1) * a.width + c] = u;
+    for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+      const float hv = row[c] * inv * (w_add + a.w[c]);
+      a.h[(size_t)t * a.width + c] = hv;
+      row[c] = hv;  // (own columns only) what the sublayer reads stays in LDS for the router below
     }
-    if (H > 0) a.canon_hist[(size_t)(H - 1) * a.width + c] = cur;
-    a.h[c] = cur + acc;
+  } else {
+    const int H = a.canon_taps - 1;  // (one token: the launcher checks)
+    for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+      const float cur = row[c] * inv * (w_add + a.w[c]);
+      const unsigned short* w = a.canon_w + (size_t)c * a.canon_taps;
+      float acc = tl_bf2f(w[H]) * cur;
+      for (int j = 0; j < H; ++j) {
+        const float u = a.canon_hist[(size_t)j * a.width + c];
+        acc += tl_bf2f(w[j]) * u;
+        if (j > 0) a.canon_hist[(size_t)(j - 1) * a.width + c] = u;
+      }
+      if (H > 0) a.canon_hist[(size_t)(H - 1) * a.width + c] = cur;
+      a.h[c] = cur + acc;
+      row[c] = cur + acc;
+    }
   }
+  if (!a.route.w) return;
+  // ---- the router of the feed-forward that reads h: logits over the row in LDS, a wave per expert in turn ----
+  __syncthreads();
+  float* z = row + ((a.width + 3) & ~3);  // [experts] (+ [experts] keys + [groups] for the group-ranked kinds)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const bool vec = (a.width & 7) == 0 && ((size_t)a.route.w & 15) == 0;
+  for (int e = wave; e < a.route.experts; e += nwaves) {
+    float sdot;
+    tl_wave_dot_rows<1>(a.route.w + (size_t)e * a.width, 0, 1, row, a.width, vec, lane, &sdot);
+    if (lane == 0) z[e] = sdot + (a.route.b ? a.route.b[e] : 0.0f);
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  int* ids = a.route.ids + (size_t)t * a.route.top;
+  float* wts = a.route.wts + (size_t)t * a.route.top;
+  if (a.route.kind == TL_ROUTE_SIGMOID_GROUPS)
+    tl_route_select_sigmoid_groups(z, z + a.route.experts, z + 2 * a.route.experts, a.route.corr, a.route.experts, a.route.top,
+                                   a.route.groups, a.route.keep, ids, wts, lane);
+  else if (a.route.kind == TL_ROUTE_SOFTMAX_GROUPS)
+    tl_route_select_groups(z, z + a.route.experts, z + 2 * a.route.experts, a.route.experts, a.route.top, a.route.groups,
+                           a.route.keep, ids, wts, lane);
+  else
+    tl_route_select(z, a.route.experts, a.route.top, ids, wts, lane);
 }
 
 constexpr int kMaxRowFloats = 16 * 1024;  // 64 KB of LDS for the staged row
@@ -428,7 +456,18 @@ int tl_launch_resid_rms(const ResidRmsArgs& a, hipStream_t s) {
   TL_REQUIRE(!a.w || a.h, "resid_rms: a norm without its output");
   TL_REQUIRE(!a.canon_w || (a.T == 1 && a.w && a.canon_taps >= 1 && (a.canon_taps == 1 || a.canon_hist)),
              "resid_rms: the convolution rides along for one token behind a norm (%d tokens, %d taps)", a.T, a.canon_taps);
-  resid_rms_kernel<<<a.T, row_threads(a.T), sizeof(float) * a.width, s>>>(a);
+  size_t lds = sizeof(float) * a.width;
+  if (a.route.w) {
+    const RouterArgs& r = a.route;
+    TL_REQUIRE(a.w && r.ids && r.wts && r.experts > 0 && r.top > 0 && r.top <= r.experts && !r.gate_w,
+               "resid_rms: bad router arguments");
+    TL_REQUIRE(r.kind == TL_ROUTE_TOP_LOGITS || (r.groups > 0 && r.experts % r.groups == 0 && r.keep > 0 && r.keep <= r.groups &&
+                                                  (long long)r.keep * (r.experts / r.groups) >= r.top),
+               "resid_rms: %d experts in %d groups, %d kept, top %d", r.experts, r.groups, r.keep, r.top);
+    lds = sizeof(float) * (((a.width + 3) & ~3) + 2 * (size_t)r.experts + (r.groups > 0 ? r.groups : 0));
+    TL_REQUIRE(lds <= 64 * 1024, "resid_rms: width %d + %d experts do not fit the staged row", a.width, r.experts);
+  }
+  resid_rms_kernel<<<a.T, row_threads(a.T), lds, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }

@@ -193,6 +193,10 @@ struct ResidRmsArgs {
   const uint16_t* canon_w;
   float* canon_hist;
   int canon_taps;
+  // optional: the router of the feed-forward that reads h rides in this launch (the finished row is in LDS): route.w != NULL ->
+  // route.ids / route.wts [T][top] as tl_launch_router writes them (route.x / T / width are ignored). Not with a convolution
+  // that is a launch of its own (the router reads what the convolution leaves).
+  RouterArgs route;
 };
 int tl_launch_resid_rms(const ResidRmsArgs& a, hipStream_t s);
 // ---- norm-first blocks: Dynamic Tanh (elementwise, no statistics) and the plain residual sum ------------------------------
@@ -393,7 +397,7 @@ struct HeadNormArgs {
   int gate_ld, gate_act;
   const float* w;        // optional [vdim] (w_per_head: [heads * vdim])
   int w_per_head;
-  float out_scale;       // 0: 1
+  float out_scale;       // (a factor of 1 has to be said: 0 gives zeros)
   int T, heads, vdim;
   float eps;
 };

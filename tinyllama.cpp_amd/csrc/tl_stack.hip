@@ -1454,6 +1454,7 @@ int delta_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T, 
     hn.gate = P + L.gate_off;
     hn.gate_ld = ld;
     hn.gate_act = 1;
+    hn.out_scale = 1.0f;
     hn.w = Wt.onorm;
     hn.T = T;
     hn.heads = sp.heads;
@@ -1505,6 +1506,7 @@ int linear_mixer(TlStack* st, Layer& L, const Layer& Wt, const float* in, int T,
   HeadNormArgs hn = {};
   hn.o = st->att;
   hn.w = Wt.onorm;
+  hn.out_scale = 1.0f;
   hn.T = T;
   hn.heads = sp.heads;
   hn.vdim = sp.vdim;
@@ -1706,7 +1708,8 @@ struct Addends {
   const float* slot_w = nullptr;
   int top = 0;
 };
-int finish_x(TlStack* st, const Addends& add, Layer* next, int which, int T, hipStream_t s) {
+// *routed (optional): set when the router of `next`'s feed-forward rode in the launch (the caller then launches none)
+int finish_x(TlStack* st, const Addends& add, Layer* next, int which, int T, hipStream_t s, bool* routed = nullptr) {
   const tl_stack_config& c = st->cfg;
   const int W = c.width;
   const Layer* Wn = next ? &st->layers[next->wsrc] : nullptr;
@@ -1731,6 +1734,12 @@ int finish_x(TlStack* st, const Addends& add, Layer* next, int which, int T, hip
   r.w = Wn ? (which == 1 ? Wn->norm1 : Wn->norm2) : nullptr;
   r.eps = c.norm_eps;
   r.h = canon ? st->hn : st->h;
+  const bool one_launch = !canon || (T == 1 && st->fuse_canon);  // h is finished by the norm's own launch
+  if (routed) *routed = false;
+  if (routed && one_launch && which == 2 && st->fuse_router && next->sp.mlp == TL_MLP_MOE && !next->sp.shared_gate) {
+    r.route = router_args(st, *next, *Wn, nullptr, T);  // the router reads the row this launch has just finished
+    *routed = true;
+  }
   if (canon && T == 1 && st->fuse_canon) {  // one token: norm, convolution and the shift of its history in the same launch
     r.h = st->h;
     r.canon_w = which == 1 ? Wn->canon1 : Wn->canon2;
@@ -1830,7 +1839,8 @@ int pre_norm_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_
     mix.b_scale = sp.side_scale;
   }
   if (sp.mlp == TL_MLP_NONE) return finish_x(st, mix, after, 1, T, s);
-  TL_TRY(finish_x(st, mix, &L, 2, T, s));
+  bool routed = false;
+  TL_TRY(finish_x(st, mix, &L, 2, T, s, &routed));
   Addends ffo;
   if (sp.mlp == TL_MLP_UNIT) {
     const int ff = sp.shared_ff;
@@ -1841,7 +1851,7 @@ int pre_norm_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_
     TL_TRY(dense_unit(st, L, Wt, st->h, T, s));
     ffo.a = st->sout;
   } else {
-    TL_TRY(tl_launch_router(router_args(st, L, Wt, st->h, T), s));
+    if (!routed) TL_TRY(tl_launch_router(router_args(st, L, Wt, st->h, T), s));
     TL_TRY(moe_experts(st, L, Wt, st->h, T, st->sout, s));
     if (T == 1 && st->gemv_decode) {
       ffo.a = st->sout;  // experts (and a shared expert) already summed with the router weights
