@@ -6,6 +6,10 @@
 //
 //   conv_kernel     grid (column blocks of 256, T): one thread per (token, channel). With one token (the decode step) the
 //                   thread is the only reader of its channel's history and shifts it in the same launch.
+//   conv4_kernel    the same for several tokens of densely packed rows when sizes allow 16-byte accesses: a thread owns four
+//                   neighbouring channels of a token (width 4096, 2048 tokens, 67 MB: 21 us against 63 us with one channel per
+//                   thread; on the q | k | v columns of a much wider product's rows it measured slower, 105 us against 63 us,
+//                   so rows that are further apart than they are wide keep the one-channel kernel).
 //   history_kernel  after a call of several tokens: the history becomes the last taps - 1 inputs (a call shorter than that
 //                   keeps the tail of the old history in front). A thread owns a channel and walks its rows in ascending order.
 #include <math.h>
@@ -37,6 +41,36 @@ __global__ __launch_bounds__(256) void conv_kernel(const ConvArgs a) {
   }
 }
 
+__global__ __launch_bounds__(256) void conv4_kernel(const ConvArgs a) {
+  const int t = blockIdx.y, c = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (c >= a.C) return;
+  const int H = a.taps - 1;
+  const float4 b = a.bias ? *reinterpret_cast<const float4*>(a.bias + c) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  const unsigned short* w = a.w + (size_t)c * a.taps;  // four rows of taps weights, one behind the other
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f), cur = acc;
+  for (int j = 0; j < a.taps; ++j) {
+    const int tt = t - H + j;
+    float4 u;
+    if (tt >= 0) {
+      u = *reinterpret_cast<const float4*>(a.in + (size_t)tt * a.ldi + c);
+      u.x += b.x, u.y += b.y, u.z += b.z, u.w += b.w;
+    } else {
+      u = *reinterpret_cast<const float4*>(a.hist + (size_t)(H + tt) * a.C + c);
+    }
+    acc.x += tl_bf2f(w[j]) * u.x;
+    acc.y += tl_bf2f(w[a.taps + j]) * u.y;
+    acc.z += tl_bf2f(w[2 * a.taps + j]) * u.z;
+    acc.w += tl_bf2f(w[3 * a.taps + j]) * u.w;
+    cur = u;
+  }
+  if (a.act == 1) {
+    acc.x = acc.x / (1.0f + expf(-acc.x)), acc.y = acc.y / (1.0f + expf(-acc.y));
+    acc.z = acc.z / (1.0f + expf(-acc.z)), acc.w = acc.w / (1.0f + expf(-acc.w));
+  }
+  if (a.add_input) acc.x += cur.x, acc.y += cur.y, acc.z += cur.z, acc.w += cur.w;
+  *reinterpret_cast<float4*>(a.out + (size_t)t * a.ldo + c) = acc;
+}
+
 __global__ __launch_bounds__(256) void conv_history_rows_kernel(const ConvArgs a) {
   const int c = blockIdx.x * 256 + threadIdx.x, H = a.taps - 1;
   if (c >= a.C) return;
@@ -56,7 +90,10 @@ int tl_launch_causal_conv(const ConvArgs& a, hipStream_t s) {
   TL_REQUIRE(a.T == 1 || a.out + (size_t)a.T * a.ldo <= a.in || a.in + (size_t)a.T * a.ldi <= a.out,
              "causal_conv: output over input with more than one token");
   TL_REQUIRE(a.act == 0 || a.act == 1, "causal_conv: activation %d", a.act);
-  conv_kernel<<<dim3((a.C + 255) / 256, a.T), 256, 0, s>>>(a);
+  const bool vec = a.T > 1 && (a.C & 3) == 0 && a.ldi == a.C && (a.ldo & 3) == 0 && ((size_t)a.in & 15) == 0 &&
+                   ((size_t)a.out & 15) == 0 && ((size_t)a.hist & 15) == 0 && ((size_t)a.bias & 15) == 0;
+  if (vec) conv4_kernel<<<dim3((a.C / 4 + 255) / 256, a.T), 256, 0, s>>>(a);
+  else conv_kernel<<<dim3((a.C + 255) / 256, a.T), 256, 0, s>>>(a);
   if (a.T > 1 && a.taps > 1) conv_history_rows_kernel<<<(a.C + 255) / 256, 256, 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
