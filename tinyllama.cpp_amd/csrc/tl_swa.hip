@@ -24,6 +24,19 @@ namespace {
 constexpr int SWA_WAVES = 4;
 constexpr int SWA_MAX_VR = 8;  // value columns per lane: vdim <= 512
 
+// cap * tanh(sc / cap) and r1 * ln(1 + r2 * d) for every score of a capped / distance-biased layer. Both are formed from the
+// hardware's exp2 / log2 / reciprocal instead of the library's tanhf / log1pf: the absolute error of a score stays near 1e-6
+// for caps of a few tens (a short series takes over below 0.1, where 1 - e^-2x would cancel), the same order as the rounding
+// of the dot product itself, and the matrix-core kernel, which pays for them on the vector unit, runs 1.3 x as fast.
+__device__ __forceinline__ float swa_cap(float sc, float cap, float inv_cap) {
+  const float x = sc * inv_cap, ax = fabsf(x), x2 = x * x;
+  const float e = __expf(-2.0f * ax);
+  const float big = copysignf(__fdividef(1.0f - e, 1.0f + e), x);
+  const float small = x * (1.0f + x2 * (-0.33333333f + x2 * (0.13333333f - 0.053968254f * x2)));
+  return cap * (ax < 0.1f ? small : big);
+}
+__device__ __forceinline__ float swa_dist(float r1, float r2, int d) { return r1 * __logf(1.0f + r2 * (float)d); }
+
 __device__ __forceinline__ void swa_st_agent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -131,8 +144,8 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
         for (int d = 0; d < a.dim; ++d) acc += qs[d] * kp[d];
       }
       sc = acc * a.scale;
-      if (a.softcap > 0.0f) sc = a.softcap * tanhf(sc / a.softcap);
-      if (a.dist_r1) sc -= r1 * log1pf(r2 * (float)(i - j));
+      if (a.softcap > 0.0f) sc = swa_cap(sc, a.softcap, 1.0f / a.softcap);
+      if (a.dist_r1) sc -= swa_dist(r1, r2, i - j);
     }
     float cm = sc;
 #pragma unroll
@@ -297,6 +310,7 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   auto clamp_row = [&](int pr) { return pr > last_q ? last_q : (pr < klo && pr >= a.keep_first) ? klo : pr; };
   const int qhs = a.q_hstride > 0 ? a.q_hstride : a.dim, khs = a.k_hstride > 0 ? a.k_hstride : a.dim;
   const float r1 = a.dist_r1 ? a.dist_r1[head] : 0.0f, r2 = a.dist_r1 ? a.dist_r2[head] : 0.0f;
+  const float inv_cap = a.softcap > 0.0f ? 1.0f / a.softcap : 0.0f;
   const bool kvec = (a.dim & 3) == 0 && (kld & 3) == 0 && (khs & 3) == 0 && ((size_t)a.kc & 15) == 0;
   const bool vvec = (a.vdim % DB) == 0 && (DB == 1 || (((size_t)a.vc & 15) == 0 && (DB != 3) && (vld % DB) == 0));
   // piece i (d = 8 i + 4 h + 0..3) of the lane's key row of a tile; rows outside [klo, last_q] are seen by no query of the
@@ -393,8 +407,8 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
       const int p = p0 + swa_acc_row(e, h);
       const bool seen = p <= qpos && (a.window <= 0 || qpos - p < a.window || p < a.keep_first);
       float sc = s[e] * a.scale;
-      if (a.softcap > 0.0f) sc = a.softcap * tanhf(sc / a.softcap);
-      if (a.dist_r1) sc -= r1 * log1pf(r2 * (float)(seen ? qpos - p : 0));
+      if (a.softcap > 0.0f) sc = swa_cap(sc, a.softcap, inv_cap);
+      if (a.dist_r1) sc -= swa_dist(r1, r2, seen ? qpos - p : 0);
       s[e] = seen ? sc : -INFINITY;
       tmax = fmaxf(tmax, s[e]);
     }
